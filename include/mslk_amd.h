@@ -1,0 +1,104 @@
+/*
+ * mslk_amd -- C ABI of the MI355X (gfx950) FP8 rowwise quantized-linear path.
+ *
+ * Every entry point is plain C: device pointers, sizes, a HIP stream handle passed as void*.
+ * Nothing is allocated, freed or synchronised inside a call; all pointers are borrowed for the
+ * duration of the call; kernels are enqueued on `stream` (NULL = the default stream) and are
+ * safe to record into a HIP graph.  Return value 0 = success; non-zero = argument or launch error,
+ * with a human-readable message available from mslk_amd_last_error() (thread-local).
+ *
+ * Data conventions (unchanged from the reference operators):
+ *   XQ  [M, K]  e4m3fn codes, row-major contiguous          (activations)
+ *   WQ  [N, K]  e4m3fn codes, row-major contiguous          (weights; i.e. B is column-major, "TN")
+ *   x_scale [M], w_scale [N]  fp32
+ *   bias [N]  fp32 or bf16, optional
+ *   Y   [M, N]  bf16, row-major contiguous:  Y = bf16( acc_fp32 * x_scale[m] * w_scale[n] + bias[n] )
+ */
+#ifndef MSLK_AMD_H_
+#define MSLK_AMD_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types of the high-precision quantizer input */
+#define MSLK_AMD_DTYPE_BF16 0
+#define MSLK_AMD_DTYPE_F16 1
+#define MSLK_AMD_DTYPE_F32 2
+
+/* bias element types */
+#define MSLK_AMD_BIAS_NONE 0
+#define MSLK_AMD_BIAS_F32 1
+#define MSLK_AMD_BIAS_BF16 2
+
+/* Library version string and the last error message of the calling thread. */
+const char* mslk_amd_version(void);
+const char* mslk_amd_last_error(void);
+
+/*
+ * Row-wise FP8 quantization.  Replaces quantize_fp8_row
+ * (reference: mslk/quantize/triton/fp8_quantize.py:319-378; bit-exact to its torch branch 356-378,
+ * whose arithmetic is: amax in the input dtype, clamp(min=1e-12[, max=*scale_ub]) in the input
+ * dtype, inv = fl32(fl32(1/amax) * 448), inf -> 1, code = e4m3fn_rne(fl32(x) * inv), scale = fl32(1/inv)).
+ *   x          [rows, K] elements of `x_dtype`, row stride `x_row_stride` elements, unit column stride
+ *   xq         [rows, K_out] e4m3fn, contiguous; K_out >= K, columns [K, K_out) are zero-filled
+ *              (K_out > K is the reference's align_rows_to padding, fp8_quantize.py:251-259)
+ *   scale      [rows] fp32
+ *   scale_ub   optional device pointer to ONE fp32 upper bound for amax (fp8_quantize.py:365-366)
+ */
+int mslk_amd_quantize_fp8_row(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t x_row_stride,
+                              void* xq, int64_t K_out, float* scale, const float* scale_ub, void* stream);
+
+/*
+ * Dense rowwise-scaled FP8 GEMM.  Replaces mslk::gemm::f8f8bf16_rowwise / f8f8bf16_rowwise_out
+ * (reference: csrc/gemm/gemm_ops.cpp:31-34; host wrapper csrc/gemm/ck/fp8_rowwise/fp8fp8bf16_rowwise_gemm.hip:499-576;
+ * math csrc/gemm/ck/fp8_rowwise/kernels/fp8_rowwise_common.h:54-82,168-204; bias semantics
+ * csrc/gemm/cutlass/f8f8bf16_rowwise/f8f8bf16_rowwise_common.cuh:150-198).
+ * M, N or K equal to 0 writes zeros to Y (fp8fp8bf16_rowwise_gemm.hip:531-534).
+ * `workspace` is only needed when mslk_amd_f8f8bf16_rowwise_workspace_bytes(M,N,K) > 0; it must be
+ * zero-filled before its first use and is left zero-filled by every call (split-K arrival counters).
+ */
+int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                              const void* bias, int bias_dtype, void* y,
+                              int64_t M, int64_t N, int64_t K,
+                              void* workspace, size_t workspace_bytes, void* stream);
+size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Grouped (MoE) rowwise FP8 GEMM over G independent problems given as host arrays of device
+ * pointers.  Replaces mslk::gemm::f8f8bf16_rowwise_grouped (TensorList API; reference:
+ * csrc/gemm/gemm_ops.cpp:37-38, csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:481-559,586-593).
+ * Group g computes Y_g[M_g, N_g] = bf16(XQ_g[M_g,K_g] . WQ_g[N_g,K_g]^T * x_scale_g[:,None] * w_scale_g[None,:]).
+ * M/N/K and the pointer arrays live in HOST memory and are consumed before the call returns.
+ * Groups with M_g == 0 are skipped; K_g == 0 writes zeros.
+ */
+int mslk_amd_f8f8bf16_rowwise_grouped(int G, const void* const* xq, const void* const* wq,
+                                      const float* const* x_scale, const float* const* w_scale,
+                                      void* const* y, const int64_t* M, const int64_t* N, const int64_t* K,
+                                      void* stream);
+
+/*
+ * Grouped GEMM over stacked tensors with DEVICE-resident group sizes (no host sync; graph-safe).
+ * Replaces mslk::gemm::f8f8bf16_rowwise_grouped_stacked (reference: csrc/gemm/gemm_ops.cpp:41-42,
+ * csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:607-655).
+ *   xq [total_M, K], wq [G, N, K], x_scale [total_M], w_scale [G, N], m_sizes int64 [G] on device,
+ *   y [total_M, N].  Rows beyond sum(m_sizes) are left untouched.
+ */
+int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, const float* x_scale,
+                                              const float* w_scale, const int64_t* m_sizes_dev, int G,
+                                              int64_t total_M, int64_t N, int64_t K, void* y, void* stream);
+
+/*
+ * Self-test helper: converts n fp32 values to e4m3fn with the same device routine the quantizer
+ * uses (hardware v_cvt_pk_fp8_f32 plus the NaN fix-up for |v| > 464).  Used by the parity tests to
+ * sweep the conversion against the oracle; no counterpart in the reference.
+ */
+int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MSLK_AMD_H_ */

@@ -1,0 +1,142 @@
+// C ABI of the library (declared in include/mslk_amd.h): argument validation, shape-class
+// dispatch, error reporting.  No allocation, no synchronisation, no host reads of device memory.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "../../include/mslk_amd.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return 1;
+}
+
+int check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return 0;
+  return fail("%s: %s", what, hipGetErrorString(e));
+}
+
+constexpr int64_t kIntMax = 2147483647;
+
+}  // namespace
+
+using namespace mslk_amd;
+
+extern "C" {
+
+const char* mslk_amd_version(void) { return "mslk_amd 0.1 (gfx950)"; }
+const char* mslk_amd_last_error(void) { return g_err; }
+
+int mslk_amd_quantize_fp8_row(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t x_row_stride,
+                              void* xq, int64_t K_out, float* scale, const float* scale_ub, void* stream) {
+  if (x_dtype < 0 || x_dtype > 2) return fail("quantize_fp8_row: unsupported input dtype code %d", x_dtype);
+  if (rows < 0 || K <= 0) return fail("quantize_fp8_row: rows must be >= 0 and K > 0 (got %lld, %lld)", (long long)rows, (long long)K);
+  if (K_out < K) return fail("quantize_fp8_row: K_out (%lld) < K (%lld)", (long long)K_out, (long long)K);
+  if (rows == 0) return 0;
+  if (rows > kIntMax) return fail("quantize_fp8_row: rows (%lld) exceeds 2^31-1", (long long)rows);
+  if (!x || !xq || !scale) return fail("quantize_fp8_row: null pointer");
+  return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub,
+                                           (hipStream_t)stream),
+                   "quantize_fp8_row launch");
+}
+
+size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+
+int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                              void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
+  if (M < 0 || N < 0 || K < 0) return fail("f8f8bf16_rowwise: negative dimension");
+  if (M > kIntMax || N > kIntMax || K > kIntMax) return fail("f8f8bf16_rowwise: dimension exceeds 2^31-1");
+  if (bias_dtype < 0 || bias_dtype > 2) return fail("f8f8bf16_rowwise: bad bias dtype code %d", bias_dtype);
+  if ((bias_dtype != 0) != (bias != nullptr)) return fail("f8f8bf16_rowwise: bias pointer and bias dtype disagree");
+  hipStream_t s = (hipStream_t)stream;
+  if (M == 0 || N == 0) return 0;
+  if (!y) return fail("f8f8bf16_rowwise: null output");
+  if (K == 0) return check_hip(launch_fill_zero_bf16((uint16_t*)y, M * N, s), "zero fill");
+  if (!xq || !wq || !x_scale || !w_scale) return fail("f8f8bf16_rowwise: null pointer");
+  GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
+                (int)M, (int)N, (int)K, bias_dtype};
+  if (skinny_supports(p)) return check_hip(launch_skinny(p, s), "skinny launch");
+  if (dense_tiled_supports(p)) return check_hip(launch_dense_tiled(p, s), "tiled launch");
+  return check_hip(launch_generic(p, s), "generic launch");
+}
+
+int mslk_amd_f8f8bf16_rowwise_grouped(int G, const void* const* xq, const void* const* wq,
+                                      const float* const* x_scale, const float* const* w_scale, void* const* y,
+                                      const int64_t* M, const int64_t* N, const int64_t* K, void* stream) {
+  if (G < 0) return fail("f8f8bf16_rowwise_grouped: negative group count");
+  hipStream_t s = (hipStream_t)stream;
+  GroupTable tab;
+  tab.count = 0;
+  tab.total_tiles = 0;
+  auto flush = [&]() -> int {
+    if (tab.count == 0) return 0;
+    int rc = check_hip(launch_grouped_tiled(tab, s), "grouped launch");
+    tab.count = 0;
+    tab.total_tiles = 0;
+    return rc;
+  };
+  for (int g = 0; g < G; ++g) {
+    if (M[g] < 0 || N[g] < 0 || K[g] < 0 || M[g] > kIntMax || N[g] > kIntMax || K[g] > kIntMax)
+      return fail("f8f8bf16_rowwise_grouped: bad dimensions in group %d", g);
+    if (M[g] == 0 || N[g] == 0) continue;
+    if (!y[g]) return fail("f8f8bf16_rowwise_grouped: null output in group %d", g);
+    if (K[g] == 0) {
+      if (int rc = check_hip(launch_fill_zero_bf16((uint16_t*)y[g], M[g] * N[g], s), "zero fill")) return rc;
+      continue;
+    }
+    if (!xq[g] || !wq[g] || !x_scale[g] || !w_scale[g]) return fail("f8f8bf16_rowwise_grouped: null pointer in group %d", g);
+    GemmProblem p{(const uint8_t*)xq[g], (const uint8_t*)wq[g], x_scale[g], w_scale[g], nullptr, (uint16_t*)y[g],
+                  (int)M[g], (int)N[g], (int)K[g], 0};
+    if (!dense_tiled_supports(p)) {  // odd K or alignment: per-group fallback
+      if (int rc = check_hip(launch_generic(p, s), "generic launch")) return rc;
+      continue;
+    }
+    GroupDesc& d = tab.g[tab.count];
+    d.xq = p.xq; d.wq = p.wq; d.xs = p.xs; d.ws = p.ws; d.y = p.y;
+    d.M = p.M; d.N = p.N; d.K = p.K;
+    d.tile_begin = tab.total_tiles;
+    const int64_t tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+    if (tab.total_tiles + tiles > kIntMax) return fail("f8f8bf16_rowwise_grouped: too many tiles");
+    tab.total_tiles += (int)tiles;
+    if (++tab.count == kMaxGroupsPerLaunch)
+      if (int rc = flush()) return rc;
+  }
+  return flush();
+}
+
+int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, const float* x_scale,
+                                              const float* w_scale, const int64_t* m_sizes_dev, int G,
+                                              int64_t total_M, int64_t N, int64_t K, void* y, void* stream) {
+  if (G < 0 || total_M < 0 || N < 0 || K < 0) return fail("f8f8bf16_rowwise_grouped_stacked: negative dimension");
+  if (total_M > kIntMax || N > kIntMax || K > kIntMax) return fail("f8f8bf16_rowwise_grouped_stacked: dimension exceeds 2^31-1");
+  hipStream_t s = (hipStream_t)stream;
+  if (G == 0 || total_M == 0 || N == 0) return 0;
+  if (!y) return fail("f8f8bf16_rowwise_grouped_stacked: null output");
+  if (K == 0) return check_hip(launch_fill_zero_bf16((uint16_t*)y, total_M * N, s), "zero fill");
+  if (!xq || !wq || !x_scale || !w_scale || !m_sizes_dev) return fail("f8f8bf16_rowwise_grouped_stacked: null pointer");
+  if (!grouped_tiled_supports((int)N, (int)K) || reinterpret_cast<uintptr_t>(xq) % 16 || reinterpret_cast<uintptr_t>(wq) % 16 ||
+      reinterpret_cast<uintptr_t>(y) % 8)
+    return fail("f8f8bf16_rowwise_grouped_stacked: K must be a multiple of 16 and XQ/WQ 16-byte aligned (K=%lld)", (long long)K);
+  return check_hip(launch_grouped_stacked((const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, m_sizes_dev, G,
+                                          total_M, (int)N, (int)K, (uint16_t*)y, s),
+                   "grouped stacked launch");
+}
+
+int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stream) {
+  if (n < 0) return fail("debug_cast_e4m3fn: negative count");
+  if (n == 0) return 0;
+  if (!in || !out) return fail("debug_cast_e4m3fn: null pointer");
+  return check_hip(launch_cast_e4m3fn(in, n, out, (hipStream_t)stream), "cast launch");
+}
+
+}  // extern "C"

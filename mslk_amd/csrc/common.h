@@ -1,0 +1,40 @@
+// Shared device/host helpers for the gfx950 FP8 rowwise kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mslk_amd {
+
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kWave = 64;
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+// fp32 -> bf16 bits, round to nearest even (finite inputs; NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return u >> 16;
+}
+
+// Two fp32 -> packed e4m3fn codes in the low 16 bits (lo = a, hi = b).
+// The hardware conversion rounds to nearest even; what it does above the largest finite
+// value depends on a mode bit, so magnitudes beyond 464 (the first value that does not round to
+// 448) are forced to the NaN code 0x7F here, which is what a non-saturating cast produces.
+__device__ __forceinline__ uint32_t cvt_pk_e4m3fn(float a, float b) {
+  uint32_t r = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xFFFFu;
+  uint32_t ua = __float_as_uint(a), ub = __float_as_uint(b);
+  if ((ua & 0x7FFFFFFFu) > 0x43E80000u) r = (r & 0xFF00u) | ((ua >> 24) & 0x80u) | 0x7Fu;
+  if ((ub & 0x7FFFFFFFu) > 0x43E80000u) r = (r & 0x00FFu) | ((((ub >> 24) & 0x80u) | 0x7Fu) << 8);
+  return r;
+}
+
+#define MSLK_AMD_DEVINL __device__ __forceinline__
+
+}  // namespace mslk_amd

@@ -1,0 +1,105 @@
+// Dense f8f8bf16_rowwise for gfx950: LDS-tiled MFMA kernel (large shapes), a generic
+// any-shape kernel, and the zero-fill used for empty problems.
+#include "gemm_tile.h"
+#include "kernels.h"
+
+namespace mslk_amd {
+namespace {
+
+constexpr int kXcds = 8;      // MI355X: 8 accelerator dies, workgroups are dealt to them round-robin
+constexpr int kGroupM = 4;    // tiles of one XCD form kGroupM-row panels (L2 reuse of the WQ panel)
+
+// Workgroup id -> tile.  Consecutive workgroup ids land on different XCDs (each with a private
+// L2), so XCD x is handed a contiguous range of the panel-ordered tile list.
+MSLK_AMD_DEVINL bool map_tile(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int ntiles = tiles_m * tiles_n;
+  const int per_xcd = (ntiles + kXcds - 1) / kXcds;
+  const int t = (bid % kXcds) * per_xcd + bid / kXcds;
+  if (t >= ntiles || bid / kXcds >= per_xcd) return false;
+  const int panel = kGroupM * tiles_n;
+  const int first_m = (t / panel) * kGroupM;
+  const int rows = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
+  tm = first_m + (t % panel) % rows;
+  tn = (t % panel) / rows;
+  return true;
+}
+
+template <int BM, int BN, int BIAS>
+__global__ __launch_bounds__(256) void dense_tiled_kernel(GemmProblem p, int tiles_m, int tiles_n) {
+  using TS = TileShape<BM, BN>;
+  __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
+  int tm, tn;
+  if (!map_tile(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  const int m0 = tm * BM, n0 = tn * BN;
+  GemmTile<TS, BIAS> tile;
+  const void* bias = nullptr;
+  if constexpr (BIAS == 1) bias = reinterpret_cast<const float*>(p.bias) + n0;
+  if constexpr (BIAS == 2) bias = reinterpret_cast<const uint16_t*>(p.bias) + n0;
+  tile.run(lds, p.xq + (int64_t)m0 * p.K, p.wq + (int64_t)n0 * p.K, p.xs + m0, p.ws + n0, bias,
+           p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K);
+}
+
+template <int BM, int BN>
+hipError_t launch_tiled_shape(const GemmProblem& p, hipStream_t s) {
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  const int ntiles = tiles_m * tiles_n;
+  const int grid = ((ntiles + kXcds - 1) / kXcds) * kXcds;
+  switch (p.bias_dtype) {
+    case 0: dense_tiled_kernel<BM, BN, 0><<<grid, 256, 0, s>>>(p, tiles_m, tiles_n); break;
+    case 1: dense_tiled_kernel<BM, BN, 1><<<grid, 256, 0, s>>>(p, tiles_m, tiles_n); break;
+    default: dense_tiled_kernel<BM, BN, 2><<<grid, 256, 0, s>>>(p, tiles_m, tiles_n); break;
+  }
+  return hipGetLastError();
+}
+
+// Any shape, no alignment requirement: one lane per output element, sequential K.
+__global__ __launch_bounds__(256) void generic_kernel(GemmProblem p) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)p.M * p.N) return;
+  const int m = (int)(idx / p.N), n = (int)(idx % p.N);
+  const uint8_t* a = p.xq + (int64_t)m * p.K;
+  const uint8_t* b = p.wq + (int64_t)n * p.K;
+  float acc = 0.f;
+  for (int k = 0; k < p.K; ++k)
+    acc += __builtin_amdgcn_cvt_f32_fp8((int)a[k], 0) * __builtin_amdgcn_cvt_f32_fp8((int)b[k], 0);
+  float v = (acc * p.xs[m]) * p.ws[n];
+  if (p.bias_dtype == 1) v += reinterpret_cast<const float*>(p.bias)[n];
+  else if (p.bias_dtype == 2) v += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]);
+  p.y[idx] = (uint16_t)f32_to_bf16_bits(v);
+}
+
+__global__ void fill_zero_kernel(uint16_t* y, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) y[i] = 0;
+}
+
+}  // namespace
+
+bool dense_tiled_supports(const GemmProblem& p) {
+  return p.K % 16 == 0 && p.K >= 16 && (int64_t)256 * p.K < (int64_t(1) << 32) &&
+         reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0 &&
+         reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
+}
+
+hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
+  if (!dense_tiled_supports(p)) return hipErrorInvalidValue;
+  // 256 x 256 tiles once they give every CU work; 128 x 128 below that.
+  const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+  if (big_tiles >= 192) return launch_tiled_shape<256, 256>(p, s);
+  return launch_tiled_shape<128, 128>(p, s);
+}
+
+hipError_t launch_generic(const GemmProblem& p, hipStream_t s) {
+  const int64_t total = (int64_t)p.M * p.N;
+  generic_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(p);
+  return hipGetLastError();
+}
+
+hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s) {
+  if (n <= 0) return hipSuccess;
+  const int64_t want = (n + 255) / 256;
+  fill_zero_kernel<<<(unsigned)(want > 4096 ? 4096 : want), 256, 0, s>>>(y, n);
+  return hipGetLastError();
+}
+
+}  // namespace mslk_amd

@@ -1,0 +1,55 @@
+// Internal launcher declarations shared between the kernel translation units and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace mslk_amd {
+
+hipError_t launch_quantize_fp8_row(const void* x, int dtype, int64_t rows, int64_t K, int64_t in_stride,
+                                   void* xq, int64_t K_out, float* scale, const float* scale_ub, hipStream_t s);
+hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t s);
+
+// One GEMM problem: Y[M,N] = bf16(XQ[M,K] . WQ[N,K]^T * xs[:,None] * ws[None,:] + bias[None,:]).
+struct GemmProblem {
+  const uint8_t* xq;
+  const uint8_t* wq;
+  const float* xs;
+  const float* ws;
+  const void* bias;   // nullptr, fp32 or bf16 according to bias_dtype
+  uint16_t* y;
+  int M, N, K;
+  int bias_dtype;     // 0 none, 1 fp32, 2 bf16
+};
+
+// Shape classes; each returns hipErrorInvalidValue when the shape is outside what it supports.
+bool dense_tiled_supports(const GemmProblem& p);
+hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s);
+bool skinny_supports(const GemmProblem& p);
+hipError_t launch_skinny(const GemmProblem& p, hipStream_t s);
+hipError_t launch_generic(const GemmProblem& p, hipStream_t s);   // any shape, slow
+hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s);
+
+// Grouped problems.  Up to kMaxGroupsPerLaunch descriptors travel in the kernel argument block.
+constexpr int kMaxGroupsPerLaunch = 64;
+struct GroupDesc {
+  const uint8_t* xq;
+  const uint8_t* wq;
+  const float* xs;
+  const float* ws;
+  uint16_t* y;
+  int M, N, K;
+  int tile_begin;     // first tile index of this group inside the launch
+};
+struct GroupTable {
+  GroupDesc g[kMaxGroupsPerLaunch];
+  int count;
+  int total_tiles;
+};
+bool grouped_tiled_supports(int N, int K);
+hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s);
+hipError_t launch_grouped_stacked(const uint8_t* xq, const uint8_t* wq, const float* xs, const float* ws,
+                                  const int64_t* m_sizes, int G, int64_t total_M, int N, int K, uint16_t* y,
+                                  hipStream_t s);
+
+}  // namespace mslk_amd

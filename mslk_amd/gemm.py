@@ -1,0 +1,251 @@
+"""`torch.ops.mslk.*` rowwise FP8 GEMM operators backed by the gfx950 HIP kernels.
+
+The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-34,37-42), so callers written
+against `torch.ops.mslk.f8f8bf16_rowwise` etc. run unchanged.  When the reference's own library has
+already defined a schema, only the GPU ("CUDA" dispatch key) kernel is replaced -- the same seam
+the reference's Python kernels use (mslk/gemm/flydsl/preshuffle_gemm.py:433-475).
+
+Validation and error messages follow the reference's ROCm host wrappers
+(csrc/gemm/ck/fp8_rowwise/fp8fp8bf16_rowwise_gemm.hip:499-550,
+ csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:481-559,607-655), except that `bias`
+is implemented (semantics of csrc/gemm/cutlass/f8f8bf16_rowwise/f8f8bf16_rowwise_common.cuh:150-198:
+per-column fp32 or bf16 bias added after both scales) instead of rejected.
+Only GPU kernels are registered: calling these ops with CPU tensors is a dispatcher error.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import List, Optional, Sequence
+
+import torch
+
+from . import _lib
+
+FP8_DTYPE = torch.float8_e4m3fn
+
+_SCHEMAS = {
+    "f8f8bf16_rowwise": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
+    "f8f8bf16_rowwise_out": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor(a!) output, Tensor? bias=None, bool use_fast_accum=True) -> ()",
+    "f8f8bf16_rowwise_grouped": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor[]",
+    "f8f8bf16_rowwise_grouped_cat": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor",
+    "f8f8bf16_rowwise_grouped_stacked": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor M_sizes) -> Tensor",
+}
+
+_library = torch.library.Library("mslk", "FRAGMENT")
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _check(cond: bool, msg: str = "") -> None:
+    if not cond:
+        raise RuntimeError(msg or "Expected condition to be true (mslk_amd argument check)")
+
+
+def _bias_args(bias: Optional[torch.Tensor], N: int, device: torch.device):
+    if bias is None:
+        return None, 0, None
+    _check(bias.device == device, "bias must be on the same device as XQ")
+    _check(bias.dtype in (torch.float32, torch.bfloat16), "Bias type must be bfloat16 or float32 if provided.")
+    _check(bias.numel() == N, f"bias must have N={N} elements, got {bias.numel()}")
+    b = bias.contiguous()
+    return b.data_ptr(), (1 if b.dtype == torch.float32 else 2), b
+
+
+def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None):
+    _check(XQ.dtype == WQ.dtype, f"XQ and WQ dtypes must match, got {XQ.dtype} vs {WQ.dtype}")
+    _check(XQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ.dtype}")
+    _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
+    _check(use_fast_accum, "AMD does not support disabling use_fast_accum.")
+    _check(XQ.is_cuda and XQ.is_contiguous(), "XQ must be a contiguous GPU tensor")
+    _check(WQ.is_cuda and WQ.is_contiguous(), "WQ must be a contiguous GPU tensor")
+    _check(XQ.dim() >= 1 and WQ.dim() == 2, "XQ must be at least 1-D and WQ 2-D")
+    N, K = WQ.shape
+    _check(XQ.shape[-1] == K, f"XQ and WQ must share K, got {XQ.shape[-1]} vs {K}")
+    M = 1
+    for d in XQ.shape[:-1]:
+        M *= d
+    _check(x_scale.numel() == M, f"x_scale must have M={M} elements, got {x_scale.numel()}")
+    _check(w_scale.numel() == N, f"w_scale must have N={N} elements, got {w_scale.numel()}")
+    _check(x_scale.device == XQ.device and w_scale.device == XQ.device and WQ.device == XQ.device,
+           "all operands must be on the same device")
+    out_sizes = tuple(XQ.shape[:-1]) + (N,)
+    if M == 0 or N == 0 or K == 0:
+        # empty problem: zeros of the output shape (fp8fp8bf16_rowwise_gemm.hip:531-534)
+        if output is not None:
+            return output
+        return torch.zeros(out_sizes, dtype=torch.bfloat16, device=XQ.device)
+    if output is not None:
+        Y = output
+        y_m = 1
+        for d in Y.shape[:-1]:
+            y_m *= d
+        _check(y_m == M and Y.shape[-1] == N, "output has the wrong shape")
+        _check(Y.dtype == torch.bfloat16, "output must be bfloat16")
+        _check(Y.is_cuda and Y.is_contiguous() and Y.device == XQ.device, "output must be a contiguous GPU tensor")
+    else:
+        Y = torch.empty(out_sizes, dtype=torch.bfloat16, device=XQ.device)
+    xs = x_scale.contiguous()
+    ws = w_scale.contiguous()
+    bias_ptr, bias_code, _keep = _bias_args(bias, N, XQ.device)
+    with torch.cuda.device(XQ.device):
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise(
+            XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
+            M, N, K, None, 0, _stream_ptr(XQ.device)))
+    return Y
+
+
+def f8f8bf16_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
+    return _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum)
+
+
+def f8f8bf16_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_accum=True):
+    _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output)
+
+
+def _check_grouped(XQ: Sequence[torch.Tensor], WQ, x_scale, w_scale):
+    _check(len(XQ) == len(WQ) == len(x_scale) == len(w_scale), "All inputs must have the same number of groups.")
+    for x in XQ:
+        _check(x.is_cuda and x.is_contiguous(), "XQ tensors must be contiguous GPU tensors")
+        _check(x.dim() == 2, "Inputs must be 2D.")
+    for w in WQ:
+        _check(w.is_cuda and w.is_contiguous(), "WQ tensors must be contiguous GPU tensors")
+        _check(w.dim() == 2, "Inputs must be 2D.")
+        _check(XQ[0].dtype == w.dtype, f"XQ and WQ dtypes must match, got {XQ[0].dtype} vs {w.dtype}")
+        _check(w.shape[0] >= 512 and w.shape[1] >= 512,
+               "N and K must be at least 512 for grouped gemm. For smaller inputs, consider unrolling.")
+    for s in list(x_scale) + list(w_scale):
+        _check(s.dtype == torch.float32, "Scales must be float32.")
+    if len(XQ):
+        _check(XQ[0].dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ[0].dtype}")
+    for x, w, xs, ws in zip(XQ, WQ, x_scale, w_scale):
+        _check(x.shape[1] == w.shape[1], "XQ and WQ of a group must share K")
+        _check(xs.numel() == x.shape[0] and ws.numel() == w.shape[0], "scale sizes must match M and N of their group")
+        _check(w.device == x.device and xs.device == x.device and ws.device == x.device and x.device == XQ[0].device,
+               "all operands must be on the same device")
+
+
+def _launch_grouped(XQ, WQ, x_scale, w_scale, outs: List[torch.Tensor]) -> None:
+    G = len(XQ)
+    xs = [s.contiguous() for s in x_scale]
+    ws = [s.contiguous() for s in w_scale]
+    PtrArr = ctypes.c_void_p * G
+    I64Arr = ctypes.c_int64 * G
+    dev = XQ[0].device
+    with torch.cuda.device(dev):
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped(
+            G, PtrArr(*[t.data_ptr() for t in XQ]), PtrArr(*[t.data_ptr() for t in WQ]),
+            PtrArr(*[t.data_ptr() for t in xs]), PtrArr(*[t.data_ptr() for t in ws]),
+            PtrArr(*[t.data_ptr() for t in outs]),
+            I64Arr(*[t.shape[0] for t in XQ]), I64Arr(*[t.shape[0] for t in WQ]), I64Arr(*[t.shape[1] for t in WQ]),
+            _stream_ptr(dev)))
+
+
+def f8f8bf16_rowwise_grouped(XQ, WQ, x_scale, w_scale) -> List[torch.Tensor]:
+    """TensorList grouped GEMM; the outputs are views into ONE flat bf16 buffer
+    (fp8_rowwise_grouped_gemm.hip:528-529,553-557)."""
+    _check_grouped(XQ, WQ, x_scale, w_scale)
+    if len(XQ) == 0:
+        return []
+    sizes = [x.shape[0] * w.shape[0] for x, w in zip(XQ, WQ)]
+    flat = torch.empty(sum(sizes), dtype=torch.bfloat16, device=XQ[0].device)
+    outs = [t.view(x.shape[0], w.shape[0]) for t, x, w in zip(flat.split(sizes), XQ, WQ)]
+    _launch_grouped(XQ, WQ, x_scale, w_scale, outs)
+    return outs
+
+
+def f8f8bf16_rowwise_grouped_cat(XQ, WQ, x_scale, w_scale) -> torch.Tensor:
+    """Same computation, outputs concatenated along M (all groups must share N)."""
+    _check_grouped(XQ, WQ, x_scale, w_scale)
+    _check(len(XQ) > 0, "at least one group is required")
+    N = WQ[0].shape[0]
+    _check(all(w.shape[0] == N for w in WQ), "all groups must share N to concatenate outputs")
+    total_M = sum(x.shape[0] for x in XQ)
+    Y = torch.empty((total_M, N), dtype=torch.bfloat16, device=XQ[0].device)
+    outs = list(Y.split([x.shape[0] for x in XQ], dim=0))
+    _launch_grouped(XQ, WQ, x_scale, w_scale, outs)
+    return Y
+
+
+def f8f8bf16_rowwise_grouped_stacked(XQ, WQ, x_scale, w_scale, M_sizes) -> torch.Tensor:
+    """XQ [total_M, K], WQ [G, N, K], x_scale [total_M], w_scale [G, N], M_sizes int64 [G] on the GPU
+    (fp8_rowwise_grouped_gemm.hip:607-655).  M_sizes is never read on the host."""
+    _check(XQ.is_cuda and XQ.is_contiguous() and WQ.is_cuda and WQ.is_contiguous(), "XQ/WQ must be contiguous GPU tensors")
+    _check(XQ.dim() == 2 and WQ.dim() == 3, "XQ must be 2-D [total_M, K] and WQ 3-D [G, N, K]")
+    _check(XQ.dtype == WQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950")
+    _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
+    _check(M_sizes.is_cuda and M_sizes.dtype == torch.int64, "M_sizes must be an int64 GPU tensor")
+    total_M, K = XQ.shape
+    G, N, Kw = WQ.shape
+    _check(K == Kw, "XQ and WQ must share K")
+    _check(M_sizes.numel() == G, "M_sizes must have one entry per group")
+    _check(x_scale.numel() == total_M and w_scale.numel() == G * N, "scale sizes must match total_M and G*N")
+    Y = torch.empty((total_M, N), dtype=torch.bfloat16, device=XQ.device)
+    if total_M == 0 or N == 0 or G == 0:
+        return Y
+    if K == 0:
+        return Y.zero_()
+    xs, ws, ms = x_scale.contiguous(), w_scale.contiguous(), M_sizes.contiguous()
+    with torch.cuda.device(XQ.device):
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped_stacked(
+            XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), ms.data_ptr(), G, total_M, N, K,
+            Y.data_ptr(), _stream_ptr(XQ.device)))
+    return Y
+
+
+# ---------------------------------------------------------------------------------------------
+# registration
+# ---------------------------------------------------------------------------------------------
+_IMPLS = {
+    "f8f8bf16_rowwise": f8f8bf16_rowwise,
+    "f8f8bf16_rowwise_out": f8f8bf16_rowwise_out,
+    "f8f8bf16_rowwise_grouped": f8f8bf16_rowwise_grouped,
+    "f8f8bf16_rowwise_grouped_cat": f8f8bf16_rowwise_grouped_cat,
+    "f8f8bf16_rowwise_grouped_stacked": f8f8bf16_rowwise_grouped_stacked,
+}
+
+
+def _fake_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
+    # mslk/gemm/_meta.py:26-50, generalised to any number of leading dims
+    return torch.empty(tuple(XQ.shape[:-1]) + (WQ.shape[0],), dtype=torch.bfloat16, device=XQ.device)
+
+
+def _fake_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_accum=True):
+    return None
+
+
+def _fake_grouped(XQ, WQ, x_scale, w_scale):
+    return [torch.empty((x.shape[0], w.shape[0]), dtype=torch.bfloat16, device=x.device) for x, w in zip(XQ, WQ)]
+
+
+def _fake_grouped_cat(XQ, WQ, x_scale, w_scale):
+    return torch.empty((sum(x.shape[0] for x in XQ), WQ[0].shape[0]), dtype=torch.bfloat16, device=XQ[0].device)
+
+
+def _fake_grouped_stacked(XQ, WQ, x_scale, w_scale, M_sizes):
+    # mslk/gemm/_meta.py:114-126
+    return torch.empty((XQ.shape[0], WQ.shape[1]), dtype=torch.bfloat16, device=XQ.device)
+
+
+_FAKES = {
+    "f8f8bf16_rowwise": _fake_rowwise,
+    "f8f8bf16_rowwise_out": _fake_rowwise_out,
+    "f8f8bf16_rowwise_grouped": _fake_grouped,
+    "f8f8bf16_rowwise_grouped_cat": _fake_grouped_cat,
+    "f8f8bf16_rowwise_grouped_stacked": _fake_grouped_stacked,
+}
+
+
+def _register() -> None:
+    for name, schema in _SCHEMAS.items():
+        already = hasattr(torch.ops.mslk, name)
+        if not already:
+            _library.define(name + schema)
+        # GPU kernel: on ROCm builds of PyTorch HIP tensors dispatch on the "CUDA" key.
+        _library.impl(name, _IMPLS[name], "CUDA", allow_override=True) if already else _library.impl(name, _IMPLS[name], "CUDA")
+        if not already:
+            torch.library.register_fake(f"mslk::{name}", _FAKES[name], lib=_library)
+
+
+_register()

@@ -1,0 +1,123 @@
+"""Row-wise FP8 quantization behind the reference's Python interface.
+
+`quantize_fp8_row` keeps the signature of the reference function
+(mslk/quantize/triton/fp8_quantize.py:319-328) and produces, on the GPU, the bits of its torch
+branch (356-378).  `quantize_fp8_per_row` is the legacy operator name for the same computation.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+FP8_DTYPE = torch.float8_e4m3fn  # gfx950 is OCP FP8 (reference: mslk/utils/device.py:135-160)
+_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor], align_rows_to: Optional[int]
+                   ) -> Tuple[torch.Tensor, torch.Tensor]:
+    if a.dtype not in _DTYPE_CODE:
+        raise RuntimeError(f"quantize_fp8_row: unsupported input dtype {a.dtype} (bf16, fp16, fp32 are supported)")
+    if a.dim() < 1:
+        raise RuntimeError("quantize_fp8_row: input must have at least one dimension")
+    if a.dim() > 4:
+        # same restriction as the reference's GPU path (fp8_quantize.py:235: "Only up to 4 dimension input tensor is supported")
+        raise RuntimeError("Only up to 4 dimension input tensor is supported if use_triton is True")
+    K = a.shape[-1]
+    if K == 0:
+        raise RuntimeError("quantize_fp8_row: cannot take the row maximum of an empty last dimension")
+    lead = a.shape[:-1]
+    rows = 1
+    for d in lead:
+        rows *= d
+    # The kernel takes one row stride; anything else (transposed views, broadcast dims) is packed first.
+    if a.stride(-1) == 1 and a.dim() == 2:
+        a2, row_stride = a, a.stride(0)
+    elif a.is_contiguous():
+        a2, row_stride = a, K
+    else:
+        a2, row_stride = a.contiguous(), K
+    K_out = K
+    if align_rows_to is not None:
+        K_out = (K + align_rows_to - 1) // align_rows_to * align_rows_to
+    xq = torch.empty(lead + (K_out,), dtype=FP8_DTYPE, device=a.device)
+    scale = torch.empty(lead, dtype=torch.float32, device=a.device)
+    ub_ptr = None
+    if scale_ub is not None:
+        scale_ub = scale_ub.to(device=a.device, dtype=torch.float32).reshape(-1)[:1].contiguous()
+        ub_ptr = scale_ub.data_ptr()
+    if rows > 0:
+        with torch.cuda.device(a.device):
+            _lib.check(_lib.lib().mslk_amd_quantize_fp8_row(
+                a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
+                scale.data_ptr(), ub_ptr, _stream_ptr(a.device)))
+    return xq, scale
+
+
+@torch.library.custom_op("mslk::quantize_fp8_row", mutates_args=(), device_types="cuda")
+def _quantize_fp8_row_op(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None,
+                         align_rows_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    return _quantize_impl(a, scale_ub, align_rows_to)
+
+
+@_quantize_fp8_row_op.register_fake
+def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None):
+    # shape function of the reference (fp8_quantize.py:381-407)
+    K = a.shape[-1]
+    if align_rows_to is not None:
+        K = (K + align_rows_to - 1) // align_rows_to * align_rows_to
+    return (torch.empty(tuple(a.shape[:-1]) + (K,), dtype=FP8_DTYPE, device=a.device),
+            torch.empty(a.shape[:-1], dtype=torch.float32, device=a.device))
+
+
+def quantize_fp8_row(
+    a: torch.Tensor,
+    scale_ub: Optional[torch.Tensor] = None,
+    zero_start_index_M: Optional[torch.Tensor] = None,
+    use_triton: bool = True,
+    output_device: Optional[torch.device] = None,
+    align_rows_to: Optional[int] = None,
+    eps_opt: Optional[float] = 1.0 / 512.0,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Quantize `a` to e4m3fn with one fp32 scale per row (reference signature, fp8_quantize.py:320-343).
+
+    Returns (a_fp8 with a's shape [last dim padded to align_rows_to], scale with shape a.shape[:-1]).
+    The numerics are those of the reference's torch branch (the contract this build is checked
+    against bit for bit): amax is clamped at 1e-12 in the input dtype, so `eps_opt` -- which only the
+    reference's Triton branch reads -- has no effect; `use_triton` is accepted and ignored (there is one
+    implementation).  `zero_start_index_M` (jagged rows) is not supported and raises.
+    The input must live on a GPU: there is no CPU implementation in this package.
+    """
+    if not a.is_cuda:
+        raise RuntimeError("mslk_amd.quantize_fp8_row: input must be a GPU tensor (no CPU implementation)")
+    if zero_start_index_M is not None:
+        raise NotImplementedError("mslk_amd.quantize_fp8_row: zero_start_index_M (jagged rows) is not supported")
+    a_fp8, a_scale = torch.ops.mslk.quantize_fp8_row(a, scale_ub, align_rows_to)
+    if output_device is not None and torch.device(output_device) != a.device:
+        a_fp8, a_scale = a_fp8.to(output_device), a_scale.to(output_device)
+    return a_fp8, a_scale
+
+
+def quantize_fp8_per_row(
+    input: torch.Tensor,
+    bs: Optional[torch.Tensor] = None,
+    scale_ub: Optional[torch.Tensor] = None,
+    output_dtype: Optional[torch.dtype] = None,
+    stochastic_rounding: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Legacy operator name for the same row-wise quantization (the reference's bench still calls the
+    path `CudaFP8Rowwise`, bench/quantize/quantize_ops.py:242-251).  `bs` and stochastic rounding
+    are not supported."""
+    if bs is not None:
+        raise NotImplementedError("quantize_fp8_per_row: `bs` is not supported")
+    if stochastic_rounding:
+        raise NotImplementedError("quantize_fp8_per_row: stochastic rounding is not supported")
+    if output_dtype is not None and output_dtype != FP8_DTYPE:
+        raise RuntimeError(f"quantize_fp8_per_row: only {FP8_DTYPE} output is supported on gfx950")
+    return quantize_fp8_row(input, scale_ub=scale_ub)

@@ -1,0 +1,122 @@
+"""CPU oracle for the FP8 rowwise quantized-linear path.  TEST INFRASTRUCTURE ONLY.
+
+Only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline leg may import this
+module.  The product package (mslk_amd) never imports it and has no CPU fallback.
+
+Every function restates, in plain CPU torch, the arithmetic of one reference function
+(paths relative to the reference checkout):
+
+  quantize_fp8_row        mslk/quantize/triton/fp8_quantize.py:356-378  (torch branch)
+  fp8 constants           mslk/utils/triton/fp8_utils.py:23-40          (e4m3fn, 448.0, 1e-12)
+  dequant_matmul          test/gemm/triton/fp8_gemm_test.py:126-132     (tight GEMM oracle)
+  matmul_fp8_row_cpu      mslk/gemm/triton/fp8_gemm.py:1186-1201        (CPU fallback = timed CPU baseline)
+  grouped_*               test/gemm/triton/grouped_gemm_test.py:116-121, bench/gemm/gemm_ops.py:632-644
+
+Pinning (what keeps this file honest; see tests/test_oracle.py):
+  * quantize: the scalar C twin in oracle/fp8_rowwise_oracle.c shares no code with torch and is
+    compared bit-for-bit, exhaustively over all 65536 bf16 inputs for many row maxima; closed
+    forms (amax = 448*2^k, zero rows, one-hot rows, -0.0, NaN rows) are asserted separately.
+  * dequant_matmul: brute-force float64 triple loop (C twin), identity / one-hot weights,
+    integer-valued codes where fp32 accumulation is exact.
+  * matmul_fp8_row_cpu: parity unpinned at bit level (it is a timing baseline whose bf16 matmul
+    rounds before scaling); it is only checked to agree with dequant_matmul within bf16 tolerance.
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import torch
+
+FP8_DTYPE = torch.float8_e4m3fn  # gfx950 uses OCP e4m3fn (mslk/utils/device.py:135-160)
+FP8_MAX = 448.0                  # torch.finfo(float8_e4m3fn).max (fp8_utils.py:40)
+EPS = 1e-12                      # fp8_utils.py:40
+
+
+def quantize_fp8_row(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None
+                     ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp8_quantize.py:360-378, CPU tensors only.
+
+    row_max is taken and clamped in the INPUT dtype (line 363-369), `448 / t` is
+    Tensor.__rdiv__ = t.reciprocal() * 448 (line 371), inf -> 1.0 (372), the product
+    a * a_scale is fp32 by type promotion (373), the cast is round-to-nearest-even with
+    no saturation (375) and the returned scale is 1 / a_scale = a_scale.reciprocal() (378).
+    """
+    assert a.device.type == "cpu"
+    a_shape = a.shape
+    row_max = torch.max(torch.abs(a), dim=-1)[0]
+    if scale_ub is not None:
+        row_max = torch.clamp(row_max, min=EPS, max=scale_ub.item())
+    else:
+        row_max = torch.clamp(row_max, min=EPS)
+    a_scale = FP8_MAX / row_max.to(torch.float32)
+    a_scale[a_scale == float("inf")] = 1.0
+    a_fp8 = (a * a_scale[..., None]).to(FP8_DTYPE)
+    return a_fp8, (1 / a_scale).view(a_shape[:-1])
+
+
+def dequantize_fp8_row(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
+    """fp32 dequantization xq * scale[:, None] (fp8_quantize.py:1140-1182 semantics)."""
+    return xq.to(torch.float32) * x_scale.to(torch.float32).reshape(*xq.shape[:-1], 1)
+
+
+def dequant_matmul(xq: torch.Tensor, wq: torch.Tensor, x_scale: torch.Tensor,
+                   w_scale: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                   dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """(xq.f32 * xs[:, None]) @ (wq.f32 * ws[:, None]).T [+ bias.f32]; no output rounding.
+
+    Same expression as test/gemm/triton/fp8_gemm_test.py:128-132.  `dtype=torch.float64`
+    gives the exact-arithmetic variant used for error budgeting.
+    """
+    x = xq.reshape(-1, xq.shape[-1]).to(dtype) * x_scale.reshape(-1, 1).to(dtype)
+    w = wq.to(dtype) * w_scale.reshape(-1, 1).to(dtype)
+    y = x @ w.T
+    if bias is not None:
+        y = y + bias.to(dtype)[None, :]
+    return y.reshape(*xq.shape[:-1], wq.shape[0])
+
+
+def matmul_fp8_row_cpu(xq: torch.Tensor, wq: torch.Tensor, x_scale: torch.Tensor,
+                       w_scale: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp8_gemm.py:1186-1201: bf16 matmul, then scale outer product, then bias, then bf16."""
+    a = xq.reshape(-1, xq.shape[-1])
+    out_shape = tuple(xq.shape[:-1]) + (wq.shape[0],)
+    if a.shape[0] == 0 or wq.shape[0] == 0 or a.shape[1] == 0:
+        return torch.zeros(out_shape, dtype=torch.bfloat16)
+    scale = x_scale.reshape(-1)[:, None] * w_scale[None, :]
+    out = torch.matmul(a.to(torch.bfloat16), wq.to(torch.bfloat16).T) * scale
+    if bias is not None:
+        out += bias[None, :]
+    return out.to(torch.bfloat16).reshape(out_shape)
+
+
+def grouped_dequant_matmul(xq: Sequence[torch.Tensor], wq: Sequence[torch.Tensor],
+                           x_scale: Sequence[torch.Tensor], w_scale: Sequence[torch.Tensor]
+                           ) -> List[torch.Tensor]:
+    """Per-group dequant_matmul (grouped_gemm_test.py:116-121 written as a loop)."""
+    return [dequant_matmul(a, b, sa, sb) for a, b, sa, sb in zip(xq, wq, x_scale, w_scale)]
+
+
+def grouped_matmul_fp8_row_cpu(xq, wq, x_scale, w_scale) -> List[torch.Tensor]:
+    """Loop of the CPU fallback over experts (bench/gemm/gemm_ops.py:632-644 pattern)."""
+    return [matmul_fp8_row_cpu(a, b, sa, sb) for a, b, sa, sb in zip(xq, wq, x_scale, w_scale)]
+
+
+# ----------------------------------------------------------------------------------------
+# error metrics used by every GEMM parity test (north_star: max-rel 1e-2, normwise 2e-3)
+# ----------------------------------------------------------------------------------------
+MAX_REL_TOL = 1e-2
+NORMWISE_TOL = 2e-3
+
+
+def gemm_errors(y: torch.Tensor, ref: torch.Tensor) -> Tuple[float, float]:
+    """(max|y-ref| / max|ref|, ||y-ref||_F / ||ref||_F) in float64."""
+    y64 = y.detach().cpu().to(torch.float64)
+    r64 = ref.detach().cpu().to(torch.float64)
+    if r64.numel() == 0:
+        return 0.0, 0.0
+    diff = (y64 - r64)
+    denom_max = r64.abs().max().item()
+    denom_f = torch.linalg.vector_norm(r64).item()
+    max_rel = diff.abs().max().item() / denom_max if denom_max > 0 else diff.abs().max().item()
+    normwise = torch.linalg.vector_norm(diff).item() / denom_f if denom_f > 0 else torch.linalg.vector_norm(diff).item()
+    return max_rel, normwise

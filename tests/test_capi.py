@@ -1,0 +1,109 @@
+"""CPU-side checks of the boundary: the shared library loads, exports every symbol the header
+declares, the operators are registered with the reference's schemas, and the shape functions and
+argument checks behave like the reference's."""
+import os
+import re
+
+import pytest
+import torch
+
+import mslk_amd
+from mslk_amd import _lib, gemm
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+F8 = torch.float8_e4m3fn
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "mslk_amd.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(mslk_amd_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    L = _lib.lib()
+    names = _declared_symbols()
+    assert len(names) >= 8
+    for n in names:
+        assert hasattr(L, n), f"{n} declared in include/mslk_amd.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert L.mslk_amd_version().decode().startswith("mslk_amd")
+    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(4096, 4096, 4096) == 0
+
+
+def test_c_abi_rejects_bad_arguments_without_a_gpu():
+    L = _lib.lib()
+    assert L.mslk_amd_quantize_fp8_row(None, 7, 1, 16, 16, None, 16, None, None, None) != 0
+    assert b"dtype" in L.mslk_amd_last_error()
+    assert L.mslk_amd_quantize_fp8_row(None, 0, 1, 16, 16, None, 8, None, None, None) != 0
+    assert b"K_out" in L.mslk_amd_last_error()
+    assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 0, None, -1, 4, 4, None, 0, None) != 0
+    assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 2, None, 4, 4, 4, None, 0, None) != 0
+    assert b"bias" in L.mslk_amd_last_error()
+    # empty problems are a successful no-op and touch no pointer
+    assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 0, None, 0, 4, 4, None, 0, None) == 0
+    assert L.mslk_amd_quantize_fp8_row(None, 0, 0, 16, 16, None, 16, None, None, None) == 0
+
+
+def test_ops_registered_with_reference_schemas():
+    s = str(torch.ops.mslk.f8f8bf16_rowwise.default._schema)
+    assert s == ("mslk::f8f8bf16_rowwise(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
+                 "Tensor? bias=None, bool use_fast_accum=True) -> Tensor")
+    s = str(torch.ops.mslk.f8f8bf16_rowwise_out.default._schema)
+    assert "Tensor(a!) output, Tensor? bias=None, bool use_fast_accum=True) -> ()" in s
+    s = str(torch.ops.mslk.f8f8bf16_rowwise_grouped.default._schema)
+    assert s == "mslk::f8f8bf16_rowwise_grouped(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor[]"
+    s = str(torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked.default._schema)
+    assert s.endswith("(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor M_sizes) -> Tensor")
+    assert hasattr(torch.ops.mslk, "quantize_fp8_row")
+
+
+def test_fake_kernels_give_reference_shapes():
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    with FakeTensorMode():
+        dev = "cuda"
+        wq = torch.empty(256, 128, dtype=F8, device=dev)
+        y = torch.ops.mslk.f8f8bf16_rowwise(torch.empty(64, 128, dtype=F8, device=dev), wq,
+                                            torch.empty(64, device=dev), torch.empty(256, device=dev))
+        assert y.shape == (64, 256) and y.dtype == torch.bfloat16
+        y = torch.ops.mslk.f8f8bf16_rowwise(torch.empty(3, 64, 128, dtype=F8, device=dev), wq,
+                                            torch.empty(3, 64, device=dev), torch.empty(256, device=dev))
+        assert y.shape == (3, 64, 256)
+        ys = torch.ops.mslk.f8f8bf16_rowwise_grouped(
+            [torch.empty(5, 512, dtype=F8, device=dev), torch.empty(0, 512, dtype=F8, device=dev)],
+            [torch.empty(512, 512, dtype=F8, device=dev)] * 2,
+            [torch.empty(5, device=dev), torch.empty(0, device=dev)], [torch.empty(512, device=dev)] * 2)
+        assert [tuple(t.shape) for t in ys] == [(5, 512), (0, 512)]
+        y = torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked(
+            torch.empty(40, 512, dtype=F8, device=dev), torch.empty(4, 768, 512, dtype=F8, device=dev),
+            torch.empty(40, device=dev), torch.empty(4, 768, device=dev), torch.empty(4, dtype=torch.int64, device=dev))
+        assert y.shape == (40, 768)
+        q, s = torch.ops.mslk.quantize_fp8_row(torch.empty(2, 3, 100, dtype=torch.bfloat16, device=dev), None, 16)
+        assert q.shape == (2, 3, 112) and q.dtype == F8 and s.shape == (2, 3) and s.dtype == torch.float32
+
+
+def test_argument_checks_raise_like_the_reference():
+    xq = torch.zeros(4, 32).to(F8)
+    wq = torch.zeros(8, 32).to(F8)
+    xs, ws = torch.ones(4), torch.ones(8)
+    with pytest.raises(RuntimeError, match="dtypes must match"):
+        gemm._rowwise_impl(xq, wq.view(torch.uint8), xs, ws, None, True)
+    with pytest.raises(RuntimeError, match="Scales must be float32"):
+        gemm._rowwise_impl(xq, wq, xs.double(), ws, None, True)
+    with pytest.raises(RuntimeError, match="use_fast_accum"):
+        gemm._rowwise_impl(xq, wq, xs, ws, None, False)
+    with pytest.raises(RuntimeError, match="same number of groups"):
+        gemm._check_grouped([xq], [wq, wq], [xs], [ws])
+    with pytest.raises(RuntimeError):
+        mslk_amd.quantize_fp8_row(torch.zeros(4, 4, dtype=torch.bfloat16))  # CPU tensor: no CPU implementation
+    with pytest.raises(NotImplementedError):
+        torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)  # no CPU kernel is registered
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "mslk_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, f

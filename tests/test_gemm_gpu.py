@@ -1,0 +1,246 @@
+"""GPU parity of f8f8bf16_rowwise against the dequantized-fp32 oracle (north_star tolerance:
+max-rel 1e-2, normwise 2e-3) plus exact textbook cases.  Shapes follow the reference's tests
+(test/gemm/gemm_test.py:204-213,354-506; test/gemm/triton/fp8_gemm_test.py:29-142)."""
+import pytest
+import torch
+
+import mslk_amd
+from mslk_amd import workloads as W
+from oracle import c_twin
+from oracle import fp8_rowwise_oracle as O
+from tests.helpers import assert_gemm_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F8 = torch.float8_e4m3fn
+
+
+def _quant_cpu(x):
+    return O.quantize_fp8_row(x)
+
+
+def _gpu(*ts):
+    return [None if t is None else t.to(DEV) for t in ts]
+
+
+def _op(xq, wq, xs, ws, bias=None):
+    y = torch.ops.mslk.f8f8bf16_rowwise(*_gpu(xq, wq, xs, ws), bias=None if bias is None else bias.to(DEV))
+    torch.cuda.synchronize()
+    return y
+
+
+def _random_problem(M, N, K, g, x_std=1.0, w_std=0.02):
+    x = (torch.randn(M, K, generator=g) * x_std).bfloat16()
+    w = (torch.randn(N, K, generator=g) * w_std).bfloat16()
+    xq, xs = _quant_cpu(x)
+    wq, ws = _quant_cpu(w)
+    return xq, wq, xs, ws
+
+
+SHAPES = [
+    # (M, N, K): reference test shapes, tile edges, K tails, odd K, skinny M
+    (256, 256, 128), (2048, 4096, 2048), (4096, 8192, 4096), (1024, 1024, 1024),
+    (300, 520, 640), (257, 255, 384), (129, 1000, 4096), (512, 768, 144), (512, 512, 16), (384, 130, 2064),
+    (100, 100, 100), (65, 33, 17), (70, 64, 1), (1, 8192, 8192), (4, 8192, 8192), (16, 8192, 8192), (64, 8192, 8192),
+    (3, 1000, 272), (17, 260, 4096), (33, 48, 512), (48, 16, 128), (64, 15, 256), (1, 1, 16), (2, 7, 24),
+]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_dense_matches_oracle(M, N, K):
+    g = torch.Generator().manual_seed(M * 1315423911 % 2**31 + N * 31 + K)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    y = _op(xq, wq, xs, ws)
+    assert y.shape == (M, N) and y.dtype == torch.bfloat16
+    assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws), f"{M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 256), (300, 260, 384), (16, 512, 512), (40, 300, 1040), (33, 20, 50)])
+def test_exact_when_fp32_accumulation_is_exact(M, N, K):
+    """Integer-valued codes in [-8, 8] and power-of-two scales: every partial sum is an integer below
+    2^24, so the fp32 result is exact in any summation order and the bf16 output must match bit for bit."""
+    g = torch.Generator().manual_seed(K)
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    xq, wq = xi.to(F8), wi.to(F8)
+    xs = 2.0 ** torch.randint(-3, 4, (M,), generator=g).float()
+    ws = 2.0 ** torch.randint(-3, 4, (N,), generator=g).float()
+    bias = torch.randint(-4, 5, (N,), generator=g).float()
+    want = ((xi @ wi.T) * xs[:, None] * ws[None, :] + bias[None, :]).bfloat16()
+    y = _op(xq, wq, xs, ws, bias)
+    assert torch.equal(y.cpu(), want)
+    small = c_twin.dequant_gemm(xq.view(torch.uint8)[:5], wq.view(torch.uint8)[:7], xs[:5], ws[:7], bias[:7])
+    assert torch.equal(y.cpu()[:5, :7].double(), small.bfloat16().double())
+
+
+def test_identity_and_one_hot_weights_select_dequantized_activations():
+    g = torch.Generator().manual_seed(9)
+    M, K = 300, 512
+    x = torch.randn(M, K, generator=g).bfloat16()
+    xq, xs = _quant_cpu(x)
+    perm = torch.randperm(K, generator=g)
+    w = torch.zeros(K, K)
+    w[torch.arange(K), perm] = 1.0
+    y = _op(xq, w.to(F8), xs, torch.ones(K))
+    want = O.dequantize_fp8_row(xq, xs)[:, perm].bfloat16()
+    assert torch.equal(y.cpu(), want)
+    # all-ones codes: every output is K * xs[m] * ws[n]
+    ones = torch.ones(64, 256).to(F8)
+    xs1, ws1 = torch.rand(64, generator=g) + 0.5, torch.rand(64, generator=g) + 0.5
+    y = _op(ones, ones, xs1, ws1)
+    assert torch.equal(y.cpu(), ((256.0 * xs1)[:, None] * ws1[None, :]).bfloat16())
+
+
+@pytest.mark.parametrize("bias_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(512, 768, 256), (16, 1024, 512), (100, 100, 100)])
+def test_bias(bias_dtype, M, N, K):
+    g = torch.Generator().manual_seed(21)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    bias = (torch.randn(N, generator=g) * 0.5).to(bias_dtype)
+    y = _op(xq, wq, xs, ws, bias)
+    assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws, bias.float()), "bias")
+    y0 = _op(xq, wq, xs, ws)
+    shift = (y.float() - y0.float()).cpu()
+    assert torch.allclose(shift, bias.float()[None, :].expand_as(shift), atol=2e-2, rtol=2e-2)
+
+
+def test_out_variant_leading_dims_and_empty():
+    g = torch.Generator().manual_seed(22)
+    xq, wq, xs, ws = _random_problem(3 * 40, 384, 256, g)
+    ref = O.dequant_matmul(xq, wq, xs, ws)
+    xq3, xs3 = xq.view(3, 40, 256), xs.view(3, 40)
+    y3 = _op(xq3, wq, xs3, ws)
+    assert y3.shape == (3, 40, 384)
+    assert_gemm_close(y3.reshape(120, 384), ref)
+    out = torch.full((3, 40, 384), 7.0, dtype=torch.bfloat16, device=DEV)
+    r = torch.ops.mslk.f8f8bf16_rowwise_out(*_gpu(xq3, wq, xs3, ws), out)
+    torch.cuda.synchronize()
+    assert r is None and torch.equal(out, y3)
+    # empty inputs give zeros of the output shape (reference test shape (0, 256, 4096) and K == 0)
+    e = torch.ops.mslk.f8f8bf16_rowwise(torch.empty(0, 256, dtype=F8, device=DEV), torch.zeros(4096, 256, device=DEV).to(F8),
+                                        torch.empty(0, device=DEV), torch.ones(4096, device=DEV))
+    assert e.shape == (0, 4096)
+    z = torch.ops.mslk.f8f8bf16_rowwise(torch.empty(5, 0, dtype=F8, device=DEV), torch.empty(9, 0, dtype=F8, device=DEV),
+                                        torch.ones(5, device=DEV), torch.ones(9, device=DEV))
+    assert z.shape == (5, 9) and (z == 0).all()
+    with pytest.raises(RuntimeError, match="use_fast_accum"):
+        torch.ops.mslk.f8f8bf16_rowwise(*_gpu(xq, wq, xs, ws), use_fast_accum=False)
+    with pytest.raises(RuntimeError, match="Scales must be float32"):
+        torch.ops.mslk.f8f8bf16_rowwise(*_gpu(xq, wq, xs.half(), ws))
+
+
+def test_unaligned_views_take_the_generic_path():
+    g = torch.Generator().manual_seed(23)
+    xq, wq, xs, ws = _random_problem(40, 72, 96, g)
+    buf = torch.empty(40 * 96 + 1, dtype=torch.uint8, device=DEV)
+    buf[1:] = xq.view(torch.uint8).reshape(-1).to(DEV)
+    xq_off = buf[1:].view(F8).view(40, 96)   # contiguous but only 1-byte aligned
+    y = torch.ops.mslk.f8f8bf16_rowwise(xq_off, *_gpu(wq, xs, ws))
+    assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws))
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 1024, 512), (16, 1024, 1024)])
+def test_hip_graph_capture_and_replay(M, N, K):
+    """The reference tests capture + replay (test/gemm/gemm_test.py:440-447); replay several times with
+    eager work in between and compare every replay with the eager result."""
+    g = torch.Generator().manual_seed(24)
+    xq, wq, xs, ws = _gpu(*_random_problem(M, N, K, g))
+    x_bf16 = torch.randn(M, K, device=DEV).bfloat16()
+    eager_q, eager_s = mslk_amd.quantize_fp8_row(x_bf16)
+    eager = torch.ops.mslk.f8f8bf16_rowwise(eager_q, wq, eager_s, ws)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            q, s = mslk_amd.quantize_fp8_row(x_bf16)
+            torch.ops.mslk.f8f8bf16_rowwise(q, wq, s, ws)
+    torch.cuda.current_stream().wait_stream(side)
+    with torch.cuda.graph(graph):
+        q, s = mslk_amd.quantize_fp8_row(x_bf16)
+        y = torch.ops.mslk.f8f8bf16_rowwise(q, wq, s, ws)
+    for _ in range(3):
+        y.fill_(0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager)
+        _ = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)  # eager work between replays
+        torch.cuda.synchronize()
+
+
+def _check_sampled(y, xq, wq, xs, ws, bias, g, rows=48, what=""):
+    """Full-size outputs are checked against the oracle on a seeded sample of rows."""
+    M = xq.shape[0]
+    idx = torch.randperm(M, generator=g)[: min(rows, M)].sort().values
+    ref = O.dequant_matmul(xq[idx].cpu(), wq.cpu(), xs[idx].cpu(), ws.cpu(), None if bias is None else bias.float().cpu())
+    return assert_gemm_close(y[idx.to(y.device)], ref, what)
+
+
+def _quantize_gpu_checked(t_cpu, g, rows=32):
+    """Quantize on the GPU and confirm a sample of rows bit-exact against the oracle."""
+    q, s = mslk_amd.quantize_fp8_row(t_cpu.to(DEV))
+    idx = torch.randperm(t_cpu.shape[0], generator=g)[: min(rows, t_cpu.shape[0])]
+    rq, rs = O.quantize_fp8_row(t_cpu[idx])
+    assert torch.equal(q[idx.to(DEV)].cpu().view(torch.uint8), rq.view(torch.uint8))
+    assert torch.equal(s[idx.to(DEV)].cpu().view(torch.int32), rs.view(torch.int32))
+    return q, s
+
+
+def test_cfg0_full():
+    wl = W.cfg0()
+    xq, xs = _quant_cpu(wl.x)
+    wq, ws = _quant_cpu(wl.w)
+    gq, gs = mslk_amd.quantize_fp8_row(wl.x.to(DEV))
+    assert torch.equal(gq.cpu().view(torch.uint8), xq.view(torch.uint8)) and torch.equal(gs.cpu().view(torch.int32), xs.view(torch.int32))
+    y = _op(xq, wq, xs, ws)
+    assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws), "cfg0")
+    # and the reference's CPU emulation path (bf16 matmul then scale) agrees within its own rounding
+    cpu = O.matmul_fp8_row_cpu(xq, wq, xs, ws)
+    max_rel, normwise = O.gemm_errors(y.float(), cpu.float())
+    assert max_rel < 2e-2 and normwise < 8e-3
+
+
+def test_cfg1_full():
+    g = torch.Generator().manual_seed(101)
+    wl = W.cfg1()
+    xq, xs = _quantize_gpu_checked(wl.x, g, rows=4096)
+    wq, ws = _quantize_gpu_checked(wl.w, g, rows=4096)
+    y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
+    torch.cuda.synchronize()
+    ref = O.dequant_matmul(xq.cpu(), wq.cpu(), xs.cpu(), ws.cpu())
+    assert_gemm_close(y, ref, "cfg1")
+
+
+def test_cfg2_full_with_bias():
+    g = torch.Generator().manual_seed(102)
+    wl = W.cfg2()
+    xq, xs = _quantize_gpu_checked(wl.x, g)
+    wq, ws = _quantize_gpu_checked(wl.w, g)
+    bias = wl.bias.to(DEV)
+    y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws, bias=bias)
+    torch.cuda.synchronize()
+    assert y.shape == (8192, 28672)
+    _check_sampled(y, xq, wq, xs, ws, bias, g, rows=64, what="cfg2")
+    # linearity in the scales (size-independent property): doubling x_scale doubles y - bias exactly in fp32,
+    # so the two bf16 outputs differ by at most one rounding
+    y2 = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs * 2, ws, bias=bias)
+    sl = slice(0, 256)
+    a = (y2[sl].float() - bias.float()[None, :]) / 2
+    b = y[sl].float() - bias.float()[None, :]
+    assert torch.allclose(a, b, rtol=1.6e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("M", [1, 4, 16, 64])
+def test_cfg3_decode(M):
+    g = torch.Generator().manual_seed(103)
+    w = W.cfg3_weight()
+    wq, ws = _quantize_gpu_checked(w, g)
+    x = W.cfg3_activations(M)
+    xq, xs = mslk_amd.quantize_fp8_row(x.to(DEV))
+    rq, rs = O.quantize_fp8_row(x)
+    assert torch.equal(xq.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs.cpu().view(torch.int32), rs.view(torch.int32))
+    y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
+    torch.cuda.synchronize()
+    assert_gemm_close(y, O.dequant_matmul(rq, wq.cpu(), rs, ws.cpu()), f"cfg3 M={M}")

@@ -1,0 +1,210 @@
+"""Pins the oracle (CPU only): the scalar C twin and the torch restatement must agree bit for bit,
+and both must satisfy what the mathematics of the format fixes independently of either."""
+import json
+import os
+
+import pytest
+import torch
+
+from oracle import c_twin
+from oracle import fp8_rowwise_oracle as O
+
+ALL_BF16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "quantize_rows.json")
+
+
+def test_c_cast_matches_torch_on_all_bf16_and_random_fp32():
+    f = ALL_BF16.float()
+    t = f.to(torch.float8_e4m3fn).view(torch.uint8)
+    c = c_twin.e4m3fn_cast(f)
+    nan = torch.isnan(f)
+    assert torch.equal(t[~nan], c[~nan])
+    assert ((t[nan] & 0x7F) == 0x7F).all() and ((c[nan] & 0x7F) == 0x7F).all()
+    g = torch.Generator().manual_seed(7)
+    x = torch.randint(-2**31, 2**31 - 1, (4_000_000,), generator=g, dtype=torch.int64).to(torch.int32).view(torch.float32)
+    nan = torch.isnan(x)
+    assert torch.equal(x.to(torch.float8_e4m3fn).view(torch.uint8)[~nan], c_twin.e4m3fn_cast(x)[~nan])
+    y = torch.rand(4_000_000, generator=g) * 1000 - 500  # dense around the representable range and the NaN edge
+    assert torch.equal(y.to(torch.float8_e4m3fn).view(torch.uint8), c_twin.e4m3fn_cast(y))
+
+
+def test_cast_known_answers():
+    # OCP FP8 E4M3: bias 7, 3 mantissa bits, max 448 = 0x7E, subnormal step 2^-9, S.1111.111 = NaN.
+    kat = [(0.0, 0x00), (-0.0, 0x80), (1.0, 0x38), (-1.0, 0xB8), (448.0, 0x7E), (-448.0, 0xFE), (2.0**-9, 0x01),
+           (2.0**-10, 0x00), (3 * 2.0**-10, 0x02), (2.0**-6, 0x08), (1.0625, 0x38), (1.1875, 0x3A), (0.875, 0x36),
+           (447.9, 0x7E), (463.9, 0x7E), (464.0, 0x7E), (464.1, 0x7F), (480.0, 0x7F), (1e9, 0x7F),
+           (float("inf"), 0x7F), (240.0, 0x77), (256.0, 0x78), (17.0, 0x58), (19.0, 0x5A)]
+    vals = torch.tensor([k for k, _ in kat], dtype=torch.float32)
+    want = torch.tensor([v for _, v in kat], dtype=torch.uint8)
+    assert torch.equal(c_twin.e4m3fn_cast(vals), want)
+    assert torch.equal(vals.to(torch.float8_e4m3fn).view(torch.uint8), want)
+
+
+def test_cast_decode_round_trip_all_codes():
+    L = c_twin.lib()
+    for code in range(256):
+        v = L.oracle_e4m3fn_to_f32(code)
+        if code & 0x7F == 0x7F:
+            assert v != v
+            continue
+        assert L.oracle_e4m3fn_from_f32(v) == code
+        assert torch.tensor([code], dtype=torch.uint8).view(torch.float8_e4m3fn).float().item() == v
+
+
+def _rows_for_amax(amax_bits_list):
+    """One row per amax: every finite bf16 value with |v| <= amax (zero-padded to a common length)."""
+    fin = ALL_BF16[torch.isfinite(ALL_BF16.float())]
+    rows = []
+    for b in amax_bits_list:
+        amax = torch.tensor([b], dtype=torch.int16).view(torch.bfloat16).float().item()
+        rows.append(fin[fin.float().abs() <= amax])
+    K = max(r.numel() for r in rows)
+    out = torch.zeros(len(rows), K, dtype=torch.bfloat16)
+    for i, r in enumerate(rows):
+        out[i, : r.numel()] = r
+    return out
+
+
+def test_quantize_c_twin_equals_torch_exhaustive_bf16():
+    # every bf16 amax in [2^-3, 2^3): 6 binades x 128 mantissas, each against every bf16 value below it
+    amax_bits = list(range(0x3E00, 0x4100))
+    for i in range(0, len(amax_bits), 96):
+        a = _rows_for_amax(amax_bits[i : i + 96])
+        q, s = O.quantize_fp8_row(a)
+        cq, cs = c_twin.quantize_rows(a)
+        assert torch.equal(q.view(torch.uint8), cq)
+        assert torch.equal(s.view(torch.int32), cs.view(torch.int32))
+
+
+def test_quantize_scales_all_positive_bf16_amax():
+    # one-element rows: every positive finite bf16 as the row maximum (incl. subnormals and bf16 max)
+    a = ALL_BF16[1:0x7F80].reshape(-1, 1).contiguous()
+    q, s = O.quantize_fp8_row(a)
+    cq, cs = c_twin.quantize_rows(a)
+    assert torch.equal(s.view(torch.int32), cs.view(torch.int32))
+    assert torch.equal(q.view(torch.uint8), cq)
+    # the element equal to the row maximum always lands on +448 once amax >= eps
+    big = a.float().reshape(-1) >= 1.01e-12
+    assert (q.view(torch.uint8).reshape(-1)[big] == 0x7E).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_quantize_c_twin_equals_torch_random(dtype):
+    g = torch.Generator().manual_seed(11)
+    for rows, K, std in [(64, 4096, 1.0), (33, 777, 30.0), (128, 1, 1.0), (1, 128, 1e-3), (7, 9000, 1.0)]:
+        a = (torch.randn(rows, K, generator=g) * std).to(dtype)
+        a[0] = 0
+        q, s = O.quantize_fp8_row(a)
+        cq, cs = c_twin.quantize_rows(a)
+        assert torch.equal(q.view(torch.uint8), cq)
+        assert torch.equal(s.view(torch.int32), cs.view(torch.int32))
+        ub = 0.75 * std
+        q, s = O.quantize_fp8_row(a, torch.tensor([ub]))
+        cq, cs = c_twin.quantize_rows(a, ub)
+        assert torch.equal(q.view(torch.uint8), cq)
+        assert torch.equal(s.view(torch.int32), cs.view(torch.int32))
+
+
+def test_quantize_closed_forms():
+    # amax = 448 * 2^k: inv = 2^-k and scale = 2^k exactly; codes are the plain e4m3 rounding of a * 2^-k
+    for k in (-4, 0, 3):
+        amax = 448.0 * 2.0**k
+        a = torch.tensor([[amax, -amax / 2, amax / 448, 0.0, -0.0, 3 * amax / 7]], dtype=torch.bfloat16)
+        for q, s in (O.quantize_fp8_row(a), c_twin.quantize_rows(a)):
+            assert s.item() == 2.0**k
+            want = (a.float() * 2.0**-k).to(torch.float8_e4m3fn).view(torch.uint8)
+            assert torch.equal(q.view(torch.uint8), want)
+            assert q.view(torch.uint8)[0, 4].item() == 0x80  # -0.0 keeps its sign
+    # zero row: amax clamps to bf16(1e-12) = 0x2B8D; all codes 0; scale = 1/(fl(1/eps)*448)
+    z = torch.zeros(1, 64, dtype=torch.bfloat16)
+    eps = torch.tensor([0x2B8D], dtype=torch.int16).view(torch.bfloat16).float()
+    assert eps.item() == 1.0018652574217413e-12
+    inv = (1.0 / eps) * 448.0
+    for q, s in (O.quantize_fp8_row(z), c_twin.quantize_rows(z)):
+        assert (q.view(torch.uint8) == 0).all()
+        assert s.item() == (1.0 / inv).item() == 2.236306529429413e-15
+    # fp16 input: 1e-12 is 0 in fp16, a zero row hits the inf -> 1.0 rule
+    zh = torch.zeros(1, 8, dtype=torch.float16)
+    for q, s in (O.quantize_fp8_row(zh), c_twin.quantize_rows(zh)):
+        assert s.item() == 1.0 and (q.view(torch.uint8) == 0).all()
+    # one-hot row: the single non-zero becomes +-448, everything else 0
+    oh = torch.zeros(1, 100, dtype=torch.bfloat16)
+    oh[0, 37] = -3.140625
+    for q, s in (O.quantize_fp8_row(oh), c_twin.quantize_rows(oh)):
+        c = q.view(torch.uint8)
+        assert c[0, 37].item() == 0xFE and c.sum().item() == 0xFE
+    # NaN anywhere in the row poisons the whole row
+    n = torch.ones(1, 16, dtype=torch.bfloat16)
+    n[0, 5] = float("nan")
+    for q, s in (O.quantize_fp8_row(n), c_twin.quantize_rows(n)):
+        assert torch.isnan(s).all() and ((q.view(torch.uint8) & 0x7F) == 0x7F).all()
+
+
+def test_quantize_invariants():
+    g = torch.Generator().manual_seed(3)
+    a = (torch.randn(256, 1024, generator=g) * torch.logspace(-6, 6, 256)[:, None]).to(torch.bfloat16)
+    q, s = O.quantize_fp8_row(a)
+    assert (s > 0).all()
+    c = q.view(torch.uint8)
+    assert ((c & 0x7F) == 0x7E).any(dim=1).all(), "every non-zero row holds a +-448 code"
+    assert ((c & 0x7F) != 0x7F).all(), "no NaN codes without scale_ub"
+    deq = q.float() * s[:, None]
+    err = (deq - a.float()).abs()
+    # half an e4m3 ulp of the scaled value, plus the rounding of inv and scale (2 ulp of fp32 each)
+    half_ulp = torch.maximum(deq.abs() * 2.0**-4, s[:, None] * 2.0**-10)
+    assert (err <= half_ulp * (1 + 1e-5) + a.float().abs() * 4e-7).all()
+    # codes are monotone in the input within a row
+    order = a.float().argsort(dim=1)
+    qs = torch.gather(q.float(), 1, order)
+    assert (qs[:, 1:] >= qs[:, :-1]).all()
+
+
+def test_dequant_matmul_against_brute_force_and_identities():
+    g = torch.Generator().manual_seed(5)
+    M, N, K = 7, 9, 37
+    xq = torch.randint(0, 256, (M, K), generator=g, dtype=torch.int64).to(torch.uint8)
+    wq = torch.randint(0, 256, (N, K), generator=g, dtype=torch.int64).to(torch.uint8)
+    xq[(xq & 0x7F) == 0x7F] = 0x10
+    wq[(wq & 0x7F) == 0x7F] = 0x10
+    xs = torch.rand(M, generator=g) + 0.5
+    ws = torch.rand(N, generator=g) * 0.01
+    bias = torch.randn(N, generator=g)
+    brute = c_twin.dequant_gemm(xq, wq, xs, ws, bias)
+    got = O.dequant_matmul(xq.view(torch.float8_e4m3fn), wq.view(torch.float8_e4m3fn), xs, ws, bias, dtype=torch.float64)
+    assert torch.allclose(got, brute, rtol=1e-12, atol=1e-12)
+    got32 = O.dequant_matmul(xq.view(torch.float8_e4m3fn), wq.view(torch.float8_e4m3fn), xs, ws, bias)
+    assert torch.allclose(got32.double(), brute, rtol=1e-4, atol=1e-4)
+    # identity weights select the dequantized activations
+    K = 16
+    eye = torch.eye(K).to(torch.float8_e4m3fn)
+    x = torch.randn(5, K, generator=g).bfloat16()
+    q, s = O.quantize_fp8_row(x)
+    y = O.dequant_matmul(q, eye, s, torch.ones(K))
+    assert torch.equal(y, O.dequantize_fp8_row(q, s))
+    # the reference's CPU fallback (bf16 matmul, scaled afterwards) agrees within bf16 rounding
+    x = torch.randn(64, 256, generator=g).bfloat16()
+    w = (torch.randn(48, 256, generator=g) * 0.02).bfloat16()
+    xq_, xs_ = O.quantize_fp8_row(x)
+    wq_, ws_ = O.quantize_fp8_row(w)
+    ref = O.dequant_matmul(xq_, wq_, xs_, ws_)
+    cpu = O.matmul_fp8_row_cpu(xq_, wq_, xs_, ws_)
+    max_rel, normwise = O.gemm_errors(cpu.float(), ref)
+    assert max_rel < 2e-2 and normwise < 8e-3
+
+
+def test_golden_quantize_rows():
+    """Vectors committed under tests/golden (made by tests/golden/make_quantize_vectors.py with plain
+    torch): guards the oracle against drift of the library routines it is written in."""
+    with open(GOLDEN) as f:
+        data = json.load(f)
+    for case in data["cases"]:
+        a = torch.tensor(case["input_bf16_bits"], dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+        ub = None if case["scale_ub"] is None else torch.tensor([case["scale_ub"]])
+        q, s = O.quantize_fp8_row(a, ub)
+        cq, cs = c_twin.quantize_rows(a, case["scale_ub"])
+        want_q = torch.tensor(case["codes"], dtype=torch.uint8)
+        want_s = torch.tensor(case["scale_bits"], dtype=torch.int32)
+        nan = want_q.new_tensor([(b & 0x7F800000) == 0x7F800000 and (b & 0x7FFFFF) != 0 for b in case["scale_bits"]]).bool()
+        for got_q, got_s in ((q.view(torch.uint8), s), (cq, cs)):
+            assert torch.equal(got_q[~nan], want_q[~nan]), case["name"]
+            assert torch.equal(got_s.view(torch.int32)[~nan], want_s[~nan]), case["name"]

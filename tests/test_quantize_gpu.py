@@ -1,0 +1,151 @@
+"""GPU parity of the HIP row quantizer against the oracle: codes and scales bit for bit.
+Shapes follow the reference's tests (test/quantize/triton/fp8_quantize_test.py:139-220,
+test/quantize/fp8_quantize_correctness_test.py:60-124)."""
+import pytest
+import torch
+
+import mslk_amd
+from mslk_amd import _lib
+from oracle import c_twin
+from oracle import fp8_rowwise_oracle as O
+from tests.helpers import assert_quant_bit_exact, bits32, codes
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+ALL_BF16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+
+
+def _run(a_cpu, scale_ub=None, align=None):
+    ub = None if scale_ub is None else scale_ub.to(DEV)
+    xq, s = mslk_amd.quantize_fp8_row(a_cpu.to(DEV), scale_ub=ub, align_rows_to=align)
+    torch.cuda.synchronize()
+    return xq, s
+
+
+def test_hw_cast_sweep_matches_oracle():
+    """Device conversion routine vs the C twin: every fp32 with a zero low mantissa half (all
+    exponents, signs, 7 mantissa bits x 512 patterns) plus dense random bits and the 448..480 edge."""
+    g = torch.Generator().manual_seed(1)
+    hi = torch.arange(65536, dtype=torch.int64)
+    lo_patterns = torch.tensor([0x0000, 0x0001, 0x7FFF, 0x8000, 0x8001, 0xFFFF, 0x4000, 0xC000], dtype=torch.int64)
+    bits = ((hi[:, None] << 16) | lo_patterns[None, :]).reshape(-1)
+    rnd = torch.randint(0, 2**32, (8_000_000,), generator=g, dtype=torch.int64)
+    edge = torch.linspace(440.0, 482.0, 200001).view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    allbits = torch.cat([bits, rnd, edge, edge | 0x80000000])
+    x = (allbits & 0xFFFFFFFF).to(torch.int64)
+    x = torch.where(x >= 2**31, x - 2**32, x).to(torch.int32).view(torch.float32)
+    out = torch.empty(x.numel(), dtype=torch.uint8, device=DEV)
+    xd = x.to(DEV)
+    _lib.check(_lib.lib().mslk_amd_debug_cast_e4m3fn(xd.data_ptr(), x.numel(), out.data_ptr(), None))
+    torch.cuda.synchronize()
+    want = c_twin.e4m3fn_cast(x)
+    got = out.cpu()
+    nan = torch.isnan(x)
+    assert torch.equal(got[~nan], want[~nan])
+    assert ((got[nan] & 0x7F) == 0x7F).all()
+
+
+def test_every_bf16_amax_and_every_bf16_value():
+    # scales: every positive finite bf16 as a one-element row (tests the device 1/x and the eps clamp)
+    a = ALL_BF16[1:0x7F80].reshape(-1, 1).contiguous()
+    xq, s = _run(a)
+    assert_quant_bit_exact(a, xq, s)
+    # codes: rows holding every finite bf16 up to amax, for a spread of amax values
+    fin = ALL_BF16[torch.isfinite(ALL_BF16.float())]
+    rows = []
+    for b in list(range(0x3F00, 0x4000, 3)) + [0x0001, 0x0080, 0x2B8D, 0x2B8E, 0x3380, 0x4700, 0x7F7F]:
+        amax = torch.tensor([b], dtype=torch.int16).view(torch.bfloat16).float().item()
+        rows.append(fin[fin.float().abs() <= amax])
+    K = (max(r.numel() for r in rows) + 7) // 8 * 8
+    a = torch.zeros(len(rows), K, dtype=torch.bfloat16)
+    for i, r in enumerate(rows):
+        a[i, : r.numel()] = r
+    xq, s = _run(a)
+    assert_quant_bit_exact(a, xq, s)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_reference_shape_sweep(dtype):
+    g = torch.Generator().manual_seed(2)
+    shapes = [(2, n) for n in range(1, 9000, 100)]
+    shapes += [(16, 16), (64, 512), (1024, 1024), (4096, 2048), (8192, 4096), (333, 777), (1, 128), (128, 1),
+               (5, 8192), (3, 16384), (2, 40000), (2, 70008), (2500, 8192), (64, 8192), (1, 8192)]
+    for shape in shapes:
+        a = torch.randn(shape, generator=g).to(dtype)
+        xq, s = _run(a)
+        assert_quant_bit_exact(a, xq, s)
+
+
+def test_special_rows_and_magnitudes():
+    g = torch.Generator().manual_seed(3)
+    a = (torch.randn(512, 2048, generator=g) * torch.logspace(-20, 20, 512)[:, None]).to(torch.bfloat16)
+    a[0] = 0
+    a[1, 5] = float("nan")
+    a[2] = -0.0
+    a[3, 100] = float("inf")
+    a[4] = 1e-39          # bf16 subnormals
+    a[5] = 3.3895313892515355e38
+    a[6, :] = 0; a[6, 77] = -5.0
+    xq, s = _run(a)
+    assert_quant_bit_exact(a, xq, s)
+    assert codes(xq)[2].eq(0x80).all()
+    assert s[0].item() == 2.236306529429413e-15
+    for dtype, zero_scale in ((torch.float16, 1.0), (torch.float32, 2.2321429389771845e-15)):
+        z = torch.zeros(4, 256, dtype=dtype)
+        xq, s = _run(z)
+        assert_quant_bit_exact(z, xq, s)
+        assert s[0].item() == zero_scale
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_scale_ub(dtype):
+    g = torch.Generator().manual_seed(4)
+    for shape in [(64, 1024), (7, 777), (2500, 4096)]:
+        a = (torch.randn(shape, generator=g) * 3).to(dtype)
+        for ub in (1200.0, 1.2345, 0.0):
+            t = torch.tensor([ub], dtype=torch.float32)
+            xq, s = _run(a, scale_ub=t)
+            assert_quant_bit_exact(a, xq, s, scale_ub=t)
+
+
+def test_batched_strided_and_padded_inputs():
+    g = torch.Generator().manual_seed(5)
+    for shape in [(3, 64, 512), (2, 3, 17, 136), (4, 1, 8)]:
+        a = torch.randn(shape, generator=g).bfloat16()
+        xq, s = _run(a)
+        assert xq.shape == a.shape and s.shape == a.shape[:-1]
+        assert_quant_bit_exact(a, xq, s)
+    base = torch.randn(300, 1000, generator=g).bfloat16()
+    for view in (base[:, :512], base[:, 8:520], base[::2, 3:77], base.t(), base[:, 1:]):
+        xq, s = _run(view)
+        assert_quant_bit_exact(view.contiguous(), xq, s)
+    for K, align in [(100, 16), (777, 8), (4096, 16), (130, 128)]:
+        a = torch.randn(33, K, generator=g).bfloat16()
+        xq, s = _run(a, align=align)
+        K_out = (K + align - 1) // align * align
+        assert_quant_bit_exact(a, xq, s, K_out=K_out)
+
+
+def test_legacy_name_and_errors():
+    a = torch.randn(8, 64).bfloat16()
+    xq, s = mslk_amd.quantize_fp8_per_row(a.to(DEV))
+    assert_quant_bit_exact(a, xq, s)
+    with pytest.raises(NotImplementedError):
+        mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=torch.zeros(8, device=DEV))
+    with pytest.raises(RuntimeError):
+        mslk_amd.quantize_fp8_row(torch.zeros(4, 0, dtype=torch.bfloat16, device=DEV))
+    xq, s = mslk_amd.quantize_fp8_row(torch.zeros(0, 64, dtype=torch.bfloat16, device=DEV))
+    assert xq.shape == (0, 64) and s.shape == (0,)
+
+
+def test_round_trip_and_full_size_properties():
+    """cfg2-sized activations (8192 x 4096 with outlier channels): bit-exact against the oracle and the
+    size-independent properties (every row holds +-448, dequantization error within half an ulp)."""
+    from mslk_amd import workloads as W
+    wl = W.cfg1(M=8192)
+    xq, s = _run(wl.x)
+    assert_quant_bit_exact(wl.x, xq, s)
+    c = codes(xq)
+    assert ((c & 0x7F) == 0x7E).any(dim=1).all()
+    deq = xq.float().cpu() * s.cpu()[:, None]
+    assert torch.allclose(deq, wl.x.float(), atol=2e-1, rtol=1e-1)  # the reference's own round-trip bound
