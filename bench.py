@@ -1,0 +1,285 @@
+"""Benchmark of the FP8 rowwise quantized-linear path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-extras]
+
+Prints ONE JSON line.  The headline (`value`) is the reference's own GEMM metric
+(bench/gemm/gemm_bench.py:490: 2*M*N*K / t of the f8f8bf16_rowwise call, quantization outside the
+timed region as in bench/gemm/gemm_ops.py:162-169) on BASELINE config 1: M=N=K=4096, x with 1 % outlier
+channels, pre-quantized w.  A step is one f8f8bf16_rowwise call through the C ABI with all operands
+resident in HBM; steps rotate over several operand sets so that consecutive calls do not find their
+inputs in the 256 MB Infinity Cache.  Extras in the same line: the quantize pass (GB/s), quantize + GEMM
+as one path, the decode sweep (M in 1,4,16,64 at N=K=8192, GB/s of algorithmic bytes), cfg0/cfg2/cfg4 GEMM
+rates, the roofline object of the dominant kernel and the CPU baseline (the reference's CPU torch path
+restated in oracle/, timed on this host's cores on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_FLOPS = 5.0e15     # MI355X dense FP8 MFMA
+PEAK_FP8_FLOPS_REF = 4.6e15  # the figure the reference's bench uses for gfx950 (bench/gemm/gemm_bench.py:61-68)
+PEAK_HBM_BPS = 8.0e12
+
+
+def _events_ms(fn, iters):
+    """Average duration of fn() in ms, HIP events on the current stream (the one kernels launch on)."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(iters):
+        fn(i)
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _median_events_ms(fn, iters, repeats=5):
+    xs = sorted(_events_ms(fn, iters) for _ in range(repeats))
+    return xs[len(xs) // 2]
+
+
+class CApi:
+    """Direct C-ABI callers (a few microseconds of host time per launch)."""
+
+    def __init__(self):
+        import torch
+        from mslk_amd import _lib
+        self.L = _lib.lib()
+        self.check = _lib.check
+        self.stream = torch.cuda.current_stream().cuda_stream
+
+    def gemm(self, xq, wq, xs, ws, y, bias=None):
+        M = xq.shape[0]
+        N, K = wq.shape
+        bcode = 0 if bias is None else (1 if bias.dtype.itemsize == 4 else 2)
+        self.check(self.L.mslk_amd_f8f8bf16_rowwise(xq.data_ptr(), wq.data_ptr(), xs.data_ptr(), ws.data_ptr(),
+                                                    None if bias is None else bias.data_ptr(), bcode, y.data_ptr(),
+                                                    M, N, K, None, 0, self.stream))
+
+    def quantize(self, x, xq, scale):
+        rows, K = x.shape
+        self.check(self.L.mslk_amd_quantize_fp8_row(x.data_ptr(), 0, rows, K, K, xq.data_ptr(), K, scale.data_ptr(),
+                                                    None, self.stream))
+
+
+def cpu_baseline(wl, budget_s=20.0):
+    """Times the reference's CPU torch path (quantize torch branch + matmul_fp8_row CPU fallback, restated in
+    oracle/) on a row sample of the same workload sized to about `budget_s` seconds of CPU work."""
+    import torch
+    from oracle import fp8_rowwise_oracle as O
+    N, K = wl.w.shape
+    wq, ws = O.quantize_fp8_row(wl.w)
+    probe_rows = 64
+    xq, xs = O.quantize_fp8_row(wl.x[:probe_rows])
+    t0 = time.perf_counter()
+    O.matmul_fp8_row_cpu(xq, wq, xs, ws)
+    probe = max(time.perf_counter() - t0, 1e-4)
+    rows = int(min(wl.x.shape[0], max(probe_rows, probe_rows * (budget_s / 3.0) / probe)))
+    rows = max(64, rows // 64 * 64)
+    x = wl.x[:rows]
+    times = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        q, s = O.quantize_fp8_row(x)
+        O.matmul_fp8_row_cpu(q, wq, s, ws, wl.bias)
+        times.append(time.perf_counter() - t0)
+    t = sorted(times)[1]
+    return {"value": 2.0 * rows * N * K / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"first {rows} of {wl.x.shape[0]} rows of x (quantize_fp8_row torch branch + bf16 matmul CPU fallback), "
+                      f"N={N}, K={K}, median of 3, {t * 1e3:.1f} ms; os.cpu_count()={os.cpu_count()}"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true")
+    ap.add_argument("--only", default="", help="profile helper: run only this piece (gemm|quantize|decode) and exit")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
+              "run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import mslk_amd  # noqa: F401
+    from mslk_amd import workloads as W
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    api = CApi()
+    extras = {}
+
+    # ---------------------------------------------------------------- cfg1: 4096^3
+    wl = W.cfg1()
+    M, K = wl.x.shape
+    N = wl.w.shape[0]
+    x_dev = wl.x.to(dev)
+    wq0, ws0 = mslk_amd.quantize_fp8_row(wl.w.to(dev))
+    xq0, xs0 = mslk_amd.quantize_fp8_row(x_dev)
+    NSETS = 6  # 6 x (16 + 16 + 32 MiB) = 384 MiB of distinct operands > 256 MB Infinity Cache
+    sets = [(xq0.clone(), wq0.clone(), xs0.clone(), ws0.clone(), torch.empty(M, N, dtype=torch.bfloat16, device=dev))
+            for _ in range(NSETS)]
+
+    def gemm_step(i):
+        xq, wq, xs, ws, y = sets[i % NSETS]
+        api.gemm(xq, wq, xs, ws, y)
+
+    if args.only in ("", "gemm"):
+        for i in range(args.warmup):
+            gemm_step(i)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        ev_start = torch.cuda.Event(enable_timing=True)
+        ev_stop = torch.cuda.Event(enable_timing=True)
+        ev_start.record()
+        for i in range(args.steps):
+            gemm_step(i)
+        ev_stop.record()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        kern_ms = ev_start.elapsed_time(ev_stop) / args.steps
+        flops = 2.0 * M * N * K
+        value = flops / (wall_ms * 1e-3) / 1e12
+        achieved = flops / (kern_ms * 1e-3) / 1e12
+        if args.only == "gemm":
+            print(json.dumps({"gemm_ms": kern_ms, "tflops": achieved}))
+            return
+    # ---------------------------------------------------------------- quantize pass (cfg1 activations)
+    xq_tmp = torch.empty(M, K, dtype=torch.float8_e4m3fn, device=dev)
+    xs_tmp = torch.empty(M, dtype=torch.float32, device=dev)
+    xsets = [x_dev.clone() for _ in range(10)]  # 10 x 32 MiB of distinct inputs
+
+    def quant_step(i):
+        api.quantize(xsets[i % len(xsets)], xq_tmp, xs_tmp)
+
+    if not args.no_extras or args.only == "quantize":
+        for i in range(10):
+            quant_step(i)
+        q_ms = _median_events_ms(quant_step, 50)
+        q_bytes = 3.0 * M * K + 4.0 * M
+        extras["quantize_cfg1"] = {"ms": q_ms, "GBps": q_bytes / (q_ms * 1e-3) / 1e9,
+                                   "frac_hbm": q_bytes / (q_ms * 1e-3) / PEAK_HBM_BPS, "bytes": q_bytes}
+        if args.only == "quantize":
+            print(json.dumps(extras))
+            return
+
+        def path_step(i):
+            xq, wq, xs, ws, y = sets[i % NSETS]
+            api.quantize(xsets[i % len(xsets)], xq, xs)
+            api.gemm(xq, wq, xs, ws, y)
+
+        for i in range(10):
+            path_step(i)
+        p_ms = _median_events_ms(path_step, 50)
+        extras["quantize_plus_gemm_cfg1"] = {"ms": p_ms, "TFLOPs": flops / (p_ms * 1e-3) / 1e12}
+    del xsets
+
+    # ---------------------------------------------------------------- decode sweep (cfg3)
+    if not args.no_extras or args.only == "decode":
+        Nd = Kd = 8192
+        wq3, ws3 = mslk_amd.quantize_fp8_row(W.cfg3_weight().to(dev))
+        wsets = [wq3.clone() for _ in range(6)]  # 6 x 64 MiB > Infinity Cache
+        decode = {}
+        for Md in (1, 4, 16, 64):
+            xd = W.cfg3_activations(Md).to(dev)
+            xq3, xs3 = mslk_amd.quantize_fp8_row(xd)
+            y3 = torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev)
+
+            def dec_step(i):
+                api.gemm(xq3, wsets[i % len(wsets)], xs3, ws3, y3)
+
+            def dec_path_step(i):
+                api.quantize(xd, xq3, xs3)
+                api.gemm(xq3, wsets[i % len(wsets)], xs3, ws3, y3)
+
+            for i in range(12):
+                dec_step(i)
+            ms = _median_events_ms(dec_step, 60)
+            ms_path = _median_events_ms(dec_path_step, 60)
+            nbytes = Nd * Kd + Md * Kd + 2.0 * Md * Nd + 4.0 * (Md + Nd)
+            decode[f"M{Md}"] = {"ms": ms, "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / PEAK_HBM_BPS,
+                                "ms_with_quantize": ms_path, "bytes": nbytes}
+        extras["decode_N8192_K8192"] = decode
+        del wsets
+        if args.only == "decode":
+            print(json.dumps(extras))
+            return
+
+    # ---------------------------------------------------------------- other configs (GEMM rate only)
+    if not args.no_extras:
+        wl0 = W.cfg0()
+        a, sa = mslk_amd.quantize_fp8_row(wl0.x.to(dev))
+        b, sb = mslk_amd.quantize_fp8_row(wl0.w.to(dev))
+        y0 = torch.empty(1024, 1024, dtype=torch.bfloat16, device=dev)
+        ms = _median_events_ms(lambda i: api.gemm(a, b, sa, sb, y0), 100)
+        extras["gemm_cfg0_1024"] = {"ms": ms, "TFLOPs": 2.0 * 1024**3 / (ms * 1e-3) / 1e12}
+
+        wl2 = W.cfg2()
+        a, sa = mslk_amd.quantize_fp8_row(wl2.x.to(dev))
+        b, sb = mslk_amd.quantize_fp8_row(wl2.w.to(dev))
+        bias2 = wl2.bias.to(dev)
+        y2 = torch.empty(8192, 28672, dtype=torch.bfloat16, device=dev)
+        for _ in range(3):
+            api.gemm(a, b, sa, sb, y2, bias2)
+        ms = _median_events_ms(lambda i: api.gemm(a, b, sa, sb, y2, bias2), 10)
+        f2 = 2.0 * 8192 * 28672 * 4096
+        extras["gemm_cfg2_8192x28672x4096_bias"] = {"ms": ms, "TFLOPs": f2 / (ms * 1e-3) / 1e12,
+                                                     "frac_mfma": f2 / (ms * 1e-3) / PEAK_FP8_FLOPS}
+        del a, b, y2, wl2
+
+        wl4 = W.cfg4()
+        xq4, xs4 = mslk_amd.quantize_fp8_row(wl4.x.to(dev))
+        wq4, ws4 = [], []
+        for w in wl4.w:
+            q, s = mslk_amd.quantize_fp8_row(w.to(dev))
+            wq4.append(q)
+            ws4.append(s)
+        xl, sl = list(xq4.split(wl4.counts)), list(xs4.split(wl4.counts))
+        for _ in range(3):
+            torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4)
+        ms = _median_events_ms(lambda i: torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4), 10)
+        f4 = 2.0 * 8192 * 8192 * 5120
+        extras["grouped_cfg4_16x8192x5120"] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12,
+                                                "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS, "counts": wl4.counts}
+        del wq4, wl4
+
+    # ---------------------------------------------------------------- CPU baseline
+    cpu = None
+    if not args.no_cpu_baseline:
+        cpu = cpu_baseline(wl)
+
+    line = {
+        "metric": "FP8 rowwise GEMM TFLOP/s @M=N=K=4096 (% FP8 peak); decode-shape HBM GB/s",
+        "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "fp8_e4m3fn x fp8_e4m3fn -> fp32 accumulate -> bf16", "data": "synthetic",
+        "config": {"workload": "cfg1: f8f8bf16_rowwise M=N=K=4096, x ~ N(0,1) with 1% K-channels x20 quantized by "
+                               "quantize_fp8_row, w ~ N(0,0.02) pre-quantized; one step = one GEMM call via the C ABI, "
+                               f"rotating over {NSETS} operand sets ({NSETS * 64} MiB); quantize timed separately (see extras)"},
+        "pct_of_fp8_peak_5.0PF": 100.0 * value * 1e12 / PEAK_FP8_FLOPS,
+        "pct_of_reference_peak_4.6PF": 100.0 * value * 1e12 / PEAK_FP8_FLOPS_REF,
+        "roofline": {"kernel": "dense_tiled_kernel<256,256> (f8f8bf16_rowwise 4096^3)", "bound": "mfma",
+                     "achieved": achieved, "peak": PEAK_FP8_FLOPS / 1e12, "unit": "TFLOP/s",
+                     "frac": achieved * 1e12 / PEAK_FP8_FLOPS, "traffic": None, "kernel_ms": kern_ms,
+                     "flops_per_launch": flops},
+        "cpu_baseline": cpu,
+        "extras": extras,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
