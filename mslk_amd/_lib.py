@@ -9,7 +9,8 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p, POINTER
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libmslk_amd.so")
+# MSLK_AMD_LIBRARY overrides the location of the built library (e.g. an out-of-tree build).
+LIB_PATH = os.environ.get("MSLK_AMD_LIBRARY") or os.path.join(_HERE, "libmslk_amd.so")
 
 _lib = None
 

@@ -125,7 +125,7 @@ int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, co
   if (K == 0) return check_hip(launch_fill_zero_bf16((uint16_t*)y, total_M * N, s), "zero fill");
   if (!xq || !wq || !x_scale || !w_scale || !m_sizes_dev) return fail("f8f8bf16_rowwise_grouped_stacked: null pointer");
   if (!grouped_tiled_supports((int)N, (int)K) || reinterpret_cast<uintptr_t>(xq) % 16 || reinterpret_cast<uintptr_t>(wq) % 16 ||
-      reinterpret_cast<uintptr_t>(y) % 8)
+      reinterpret_cast<uintptr_t>(y) % 16)
     return fail("f8f8bf16_rowwise_grouped_stacked: K must be a multiple of 16 and XQ/WQ 16-byte aligned (K=%lld)", (long long)K);
   return check_hip(launch_grouped_stacked((const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, m_sizes_dev, G,
                                           total_M, (int)N, (int)K, (uint16_t*)y, s),

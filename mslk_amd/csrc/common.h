@@ -37,4 +37,12 @@ __device__ __forceinline__ uint32_t cvt_pk_e4m3fn(float a, float b) {
 
 #define MSLK_AMD_DEVINL __device__ __forceinline__
 
+// Two fp32 -> packed bf16 (lo = a, hi = b), round to nearest even, by the hardware conversion.
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  f32x2_t v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
+
 }  // namespace mslk_amd

@@ -78,7 +78,7 @@ __global__ void fill_zero_kernel(uint16_t* y, int64_t n) {
 bool dense_tiled_supports(const GemmProblem& p) {
   return p.K % 16 == 0 && p.K >= 16 && (int64_t)256 * p.K < (int64_t(1) << 32) &&
          reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0 &&
-         reinterpret_cast<uintptr_t>(p.y) % 8 == 0;
+         reinterpret_cast<uintptr_t>(p.y) % 16 == 0;
 }
 
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
@@ -102,4 +102,9 @@ hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s) {
   return hipGetLastError();
 }
 
+#ifdef MSLK_EXP_TRACE
+extern "C" int mslk_exp_read_trace(unsigned long long* out, int n) {
+  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), n * sizeof(unsigned long long));
+}
+#endif
 }  // namespace mslk_amd

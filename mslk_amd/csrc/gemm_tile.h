@@ -52,6 +52,24 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
 }
 
+#ifdef MSLK_EXP_TRACE
+__device__ unsigned long long g_trace[4096];
+#define MSLK_TILE_TRACE(slot)                                                            \
+  do {                                                                                   \
+    if (threadIdx.x == 0 && blockIdx.x == 0 && (slot) < 4096) g_trace[slot] = __builtin_amdgcn_s_memtime(); \
+  } while (0)
+#else
+#define MSLK_TILE_TRACE(slot) do {} while (0)
+#endif
+#ifdef MSLK_EXP_TRACE
+#define MSLK_TILE_TRACE_RT(slot)                                                         \
+  do {                                                                                   \
+    if (threadIdx.x == 0 && blockIdx.x == 0) g_trace[slot] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#else
+#define MSLK_TILE_TRACE_RT(slot) do {} while (0)
+#endif
+
 template <typename TS, int BIAS>
 struct GemmTile {
   // Per-lane state that is constant over the K loop.
@@ -81,15 +99,23 @@ struct GemmTile {
     }
   }
 
-  // Issue the DMA loads of a full K step (128 valid bytes per row) starting at byte k0 into `stage`.
+  // Wave index as a scalar, so that LDS destinations of the DMA are formed in SGPRs.
+  MSLK_AMD_DEVINL static int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
+
+  // DMA load number i (0 .. LA-1 for the XQ tile, 0 .. LB-1 for the WQ tile) of the K step at byte k0.
+  MSLK_AMD_DEVINL void issue_a(char* stage, int k0, int i) {
+    dma16(a_base + k0 + a_off[i], stage + (wave_id() * TS::LA + i) * 1024);
+  }
+  MSLK_AMD_DEVINL void issue_b(char* stage, int k0, int i) {
+    dma16(b_base + k0 + b_off[i], stage + TS::A_BYTES + (wave_id() * TS::LB + i) * 1024);
+  }
+
+  // All DMA loads of a full K step (128 valid bytes per row) starting at byte k0 into `stage`.
   MSLK_AMD_DEVINL void issue_loads(char* stage, int k0) {
-    const int wave = threadIdx.x >> 6;
 #pragma unroll
-    for (int i = 0; i < TS::LA; ++i)
-      dma16(a_base + k0 + a_off[i], stage + (wave * TS::LA + i) * 1024);
+    for (int i = 0; i < TS::LA; ++i) issue_a(stage, k0, i);
 #pragma unroll
-    for (int i = 0; i < TS::LB; ++i)
-      dma16(b_base + k0 + b_off[i], stage + TS::A_BYTES + (wave * TS::LB + i) * 1024);
+    for (int i = 0; i < TS::LB; ++i) issue_b(stage, k0, i);
   }
 
   // K tail (K % 128 != 0, K % 16 == 0): only `k_valid` bytes of each row remain.  Chunks at or
@@ -114,39 +140,92 @@ struct GemmTile {
     }
   }
 
-  // One K step of MFMAs out of `stage`.
-  MSLK_AMD_DEVINL void compute(const char* stage, v4f (&acc)[TS::FN][TS::FM]) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
+  // LDS byte offsets of this lane's two 16-byte halves of an MFMA operand fragment, relative to the
+  // first row of the fragment: lane (i = l & 15, g = l >> 4) reads logical chunks 2g and 2g + 1 of row i.
+  struct FragOff { int off0, off1; };
+  MSLK_AMD_DEVINL static FragOff frag_off() {
+    const int lane = threadIdx.x & 63;
     const int i = lane & 15, g = lane >> 4;
     const int s = lds_swz(i);
-    const int off0 = i * kBK + (((2 * g) ^ s) << 4);
-    const int off1 = i * kBK + (((2 * g + 1) ^ s) << 4);
-    const char* a_tile = stage + wm * (TS::kBM / 2) * kBK;
-    const char* b_tile = stage + TS::A_BYTES + wn * (TS::kBN / 2) * kBK;
-    v8i xf[TS::FM];
+    return FragOff{i * kBK + (((2 * g) ^ s) << 4), i * kBK + (((2 * g + 1) ^ s) << 4)};
+  }
+  MSLK_AMD_DEVINL static v8i load_frag(const char* tile, int t, FragOff fo) {
+    const v4i lo = *reinterpret_cast<const v4i*>(tile + t * 16 * kBK + fo.off0);
+    const v4i hi = *reinterpret_cast<const v4i*>(tile + t * 16 * kBK + fo.off1);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+  MSLK_AMD_DEVINL static const char* a_tile_of(const char* stage) {
+    return stage + (wave_id() >> 1) * (TS::kBM / 2) * kBK;
+  }
+  MSLK_AMD_DEVINL static const char* b_tile_of(const char* stage) {
+    return stage + TS::A_BYTES + (wave_id() & 1) * (TS::kBN / 2) * kBK;
+  }
+  // First fragments of a K step: all XQ fragments and WQ fragment 0.
+  MSLK_AMD_DEVINL void load_first_frags(const char* stage, v8i (&xf)[TS::FM], v8i& wf0) {
+    const FragOff fo = frag_off();
+    wf0 = load_frag(b_tile_of(stage), 0, fo);
 #pragma unroll
-    for (int tm = 0; tm < TS::FM; ++tm) {
-      const v4i lo = *reinterpret_cast<const v4i*>(a_tile + tm * 16 * kBK + off0);
-      const v4i hi = *reinterpret_cast<const v4i*>(a_tile + tm * 16 * kBK + off1);
-      xf[tm] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-    }
+    for (int tm = 0; tm < TS::FM; ++tm) xf[tm] = load_frag(a_tile_of(stage), tm, fo);
+  }
+
+  // One K step of MFMAs out of stage `cur`; xf / wf0 (its XQ fragments and WQ fragment 0) are
+  // already in registers.  The step is software-pipelined across the workgroup barrier:
+  //   * DMA: the global -> LDS loads of the FOLLOWING K step (byte offset k_next, stage `nxt`) are issued
+  //     between the MFMA groups of the first half of the step, so that their issue cost hides under
+  //     matrix work and they have half a step to land;
+  //   * NEXT: before the last MFMA group the wave waits for its DMA and all its LDS reads and passes the
+  //     barrier (after which stage `nxt` is complete and nobody reads `cur` any more).  The operands of
+  //     the last group are in registers; each XQ fragment is re-loaded from `nxt` right after the MFMA
+  //     that used it last, so the barrier and the LDS latency overlap with matrix work and the
+  //     following step starts with its first fragments already on their way.
+  template <bool DMA, bool NEXT>
+  MSLK_AMD_DEVINL void step(const char* cur, char* nxt, int k_next, v4f (&acc)[TS::FN][TS::FM],
+                            v8i (&xf)[TS::FM], v8i& wf0) {
+    constexpr int HALF = TS::FN / 2;
+    static_assert(TS::LA % HALF == 0 && TS::LB % HALF == 0, "DMA loads spread evenly over the first half");
+    constexpr int PA = TS::LA / HALF, PB = TS::LB / HALF;
+    const FragOff fo = frag_off();
+    const char* b_tile = b_tile_of(cur);
+    v8i wf = wf0;
 #pragma unroll
-    for (int tn = 0; tn < TS::FN; ++tn) {
-      const v4i lo = *reinterpret_cast<const v4i*>(b_tile + tn * 16 * kBK + off0);
-      const v4i hi = *reinterpret_cast<const v4i*>(b_tile + tn * 16 * kBK + off1);
-      const v8i wf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    for (int tn = 0; tn < TS::FN - 1; ++tn) {
+      const v8i wf_next = load_frag(b_tile, tn + 1, fo);
+      if constexpr (DMA) {
+        if (tn < HALF) {
+#pragma unroll
+          for (int u = 0; u < PA; ++u) issue_a(nxt, k_next, tn * PA + u);
+#pragma unroll
+          for (int u = 0; u < PB; ++u) issue_b(nxt, k_next, tn * PB + u);
+        }
+      }
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm)
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+      wf = wf_next;
+      __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (NEXT) {
+      __syncthreads();  // s_waitcnt vmcnt(0) lgkmcnt(0); s_barrier
+      wf0 = load_frag(b_tile_of(nxt), 0, fo);
+    }
+    const char* a_next = a_tile_of(nxt);
+#pragma unroll
+    for (int tm = 0; tm < TS::FM; ++tm) {
+      acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+      if constexpr (NEXT) {
+        xf[tm] = load_frag(a_next, tm, fo);
+        __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);
   }
 
   // Whole tile: K loop + epilogue.  m_rem / n_rem = valid rows / columns of this tile (>= 1).
-  // y, xs point at row m0; ws, bias, and the column offset of y at n0 are applied by the caller
-  // through y (= Y + m0 * N + n0), ws (= w_scale + n0) and bias (+ n0).
+  // xq_tile / wq_tile / xs / ws / bias / y are already offset to the tile's first row and column.
   MSLK_AMD_DEVINL void run(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, const float* xs,
                            const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K) {
+    MSLK_TILE_TRACE(140);
+    MSLK_TILE_TRACE_RT(141);
     init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, K);
     v4f acc[TS::FN][TS::FM];
 #pragma unroll
@@ -154,71 +233,106 @@ struct GemmTile {
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    const int KT = K / kBK;          // full steps
+    char* cur = lds;
+    char* nxt = lds + TS::STAGE_BYTES;
+    const int KT = K / kBK;           // full steps
     const int k_tail = K - KT * kBK;  // 0 or a multiple of 16
-    if (KT > 0) issue_loads(lds, 0);
-    for (int kt = 0; kt < KT; ++kt) {
-      // Every wave has waited for its own DMA before the barrier, so after it the whole stage
-      // kt & 1 is in LDS and nobody still reads the other stage (it was consumed in step kt - 1).
-      wait_vmcnt0();
+    v8i xf[TS::FM], wf0;
+    if (KT > 0) {
+      issue_loads(cur, 0);
       __syncthreads();
-      if (kt + 1 < KT) issue_loads(lds + ((kt + 1) & 1) * TS::STAGE_BYTES, (kt + 1) * kBK);
-      compute(lds + (kt & 1) * TS::STAGE_BYTES, acc);
+      load_first_frags(cur, xf, wf0);
+      for (int kt = 0; kt < KT - 1; ++kt) {
+        MSLK_TILE_TRACE(kt * 4 + 0);
+        step<true, true>(cur, nxt, (kt + 1) * kBK, acc, xf, wf0);
+        char* t = cur; cur = nxt; nxt = t;
+      }
+      step<false, false>(cur, nxt, 0, acc, xf, wf0);
+      { char* t = cur; cur = nxt; nxt = t; }
     }
     if (k_tail > 0) {
-      char* stage = lds + (KT & 1) * TS::STAGE_BYTES;
+      __syncthreads();   // everybody is done reading `cur` (consumed two steps ago) before it is refilled
+      issue_loads_tail(cur, KT * kBK, k_tail);
       __syncthreads();
-      issue_loads_tail(stage, KT * kBK, k_tail);
-      wait_vmcnt0();
-      __syncthreads();
-      compute(stage, acc);
+      load_first_frags(cur, xf, wf0);
+      step<false, false>(cur, nxt, 0, acc, xf, wf0);
     }
-    epilogue(acc, xs, ws, bias, y, m_rem, n_rem, N);
+    MSLK_TILE_TRACE(32 * 4 + 0);
+    __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
+    epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+    MSLK_TILE_TRACE(32 * 4 + 1);
+    MSLK_TILE_TRACE_RT(142);
   }
 
-  MSLK_AMD_DEVINL void epilogue(v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws, const void* bias,
-                                uint16_t* y, int m_rem, int n_rem, int N) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  // Epilogue.  A lane's accumulators of one 16-row m fragment are 4 consecutive n in each of the
+  // FN n fragments; storing them directly would write 32-byte pieces of 16 different rows per
+  // instruction.  Instead each wave scales, converts to bf16 and parks the 16 x (BN/2) block in a
+  // private LDS buffer (row pitch BN + 16 bytes keeps the 8-byte writes and 16-byte reads off shared
+  // banks), then reads it back row-major so that one store instruction writes 4 full rows of
+  // BN/2 bf16 (16 lanes x 16 bytes each).
+  MSLK_AMD_DEVINL void epilogue(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
+                                const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
+    constexpr int WN = TS::kBN / 2;              // columns per wave
+    constexpr int PITCH = WN * 2 + 16;           // bytes per staged row
+    constexpr int BUF = 16 * PITCH;
+    constexpr int CH = WN / 8;                   // 16-byte chunks per row (16 for BN = 256)
+    constexpr int RPI = 64 / CH;                 // rows written per store instruction
+    const int lane = threadIdx.x & 63, wave = wave_id();
     const int wm = wave >> 1, wn = wave & 1;
-    const int mi = wm * (TS::kBM / 2) + (lane & 15);
-    const int ni = wn * (TS::kBN / 2) + 4 * (lane >> 4);
-    const bool vec_store = (N & 3) == 0;
-    float xsv[TS::FM];
+    const int j = lane & 15, q = lane >> 4;
+    char* buf = lds + wave * 2 * BUF;
+    const int n_base = wn * WN;
+    const int m_base = wm * (TS::kBM / 2);
+    const bool vec_store = (N & 7) == 0;
+
+    float wsv[TS::FN][4], bv[TS::FN][4];
 #pragma unroll
-    for (int tm = 0; tm < TS::FM; ++tm) {
-      const int m = mi + tm * 16;
-      xsv[tm] = m < m_rem ? xs[m] : 0.f;
-    }
-#pragma unroll
-    for (int tn = 0; tn < TS::FN; ++tn) {
-      const int n = ni + tn * 16;
-      float wsv[4], bv[4];
+    for (int tn = 0; tn < TS::FN; ++tn)
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const bool ok = n + r < n_rem;
-        wsv[r] = ok ? ws[n + r] : 0.f;
-        if constexpr (BIAS == 1) bv[r] = ok ? reinterpret_cast<const float*>(bias)[n + r] : 0.f;
-        else if constexpr (BIAS == 2) bv[r] = ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(bias)[n + r]) : 0.f;
-        else bv[r] = 0.f;
+        const int n = n_base + tn * 16 + 4 * q + r;
+        const bool ok = n < n_rem;
+        wsv[tn][r] = ok ? ws[n] : 0.f;
+        if constexpr (BIAS == 1) bv[tn][r] = ok ? reinterpret_cast<const float*>(bias)[n] : 0.f;
+        else if constexpr (BIAS == 2) bv[tn][r] = ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(bias)[n]) : 0.f;
+        else bv[tn][r] = 0.f;
       }
+
+    const int rd_row = lane / CH, rd_chunk = lane % CH;
 #pragma unroll
-      for (int tm = 0; tm < TS::FM; ++tm) {
-        const int m = mi + tm * 16;
-        if (m >= m_rem) continue;
-        uint32_t h[4];
+    for (int tm = 0; tm < TS::FM; ++tm) {
+      char* b = buf + (tm & 1) * BUF;
+      const int m = m_base + tm * 16 + j;
+      const float xsv = m < m_rem ? xs[m] : 0.f;
+#pragma unroll
+      for (int tn = 0; tn < TS::FN; ++tn) {
+        float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          float v = (acc[tn][tm][r] * xsv[tm]) * wsv[r];
-          if constexpr (BIAS != 0) v += bv[r];
-          h[r] = f32_to_bf16_bits(v);
+          v[r] = (acc[tn][tm][r] * xsv) * wsv[tn][r];
+          if constexpr (BIAS != 0) v[r] += bv[tn][r];
         }
-        uint16_t* dst = y + (int64_t)m * N + n;
-        if (vec_store && n + 3 < n_rem) {
-          *reinterpret_cast<uint2*>(dst) = make_uint2(h[0] | (h[1] << 16), h[2] | (h[3] << 16));
-        } else {
+        uint2 pk;
+        pk.x = pack_bf16x2(v[0], v[1]);
+        pk.y = pack_bf16x2(v[2], v[3]);
+        *reinterpret_cast<uint2*>(b + j * PITCH + (tn * 16 + 4 * q) * 2) = pk;
+      }
+      // the buffer is private to the wave: LDS operations of one wave complete in order
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (n + r < n_rem) dst[r] = (uint16_t)h[r];
+      for (int pass = 0; pass < 16 / RPI; ++pass) {
+        const int row = pass * RPI + rd_row;
+        const uint4 val = *reinterpret_cast<const uint4*>(b + row * PITCH + rd_chunk * 16);
+        const int mm = m_base + tm * 16 + row;
+        const int nn = n_base + rd_chunk * 8;
+        if (mm >= m_rem || nn >= n_rem) continue;
+        uint16_t* dst = y + (int64_t)mm * N + nn;
+        if (vec_store && nn + 7 < n_rem) {
+          *reinterpret_cast<uint4*>(dst) = val;
+        } else {
+          const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            if (nn + e < n_rem) dst[e] = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
         }
       }
     }
