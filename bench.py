@@ -137,6 +137,7 @@ def main():
         xq, wq, xs, ws, y = sets[i % NSETS]
         api.gemm(xq, wq, xs, ws, y)
 
+    flops = 2.0 * M * N * K
     if args.only in ("", "gemm"):
         for i in range(args.warmup):
             gemm_step(i)
@@ -151,7 +152,6 @@ def main():
         torch.cuda.synchronize()
         wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
         kern_ms = ev_start.elapsed_time(ev_stop) / args.steps
-        flops = 2.0 * M * N * K
         value = flops / (wall_ms * 1e-3) / 1e12
         achieved = flops / (kern_ms * 1e-3) / 1e12
         if args.only == "gemm":
@@ -165,7 +165,7 @@ def main():
     def quant_step(i):
         api.quantize(xsets[i % len(xsets)], xq_tmp, xs_tmp)
 
-    if not args.no_extras or args.only == "quantize":
+    if (not args.no_extras and args.only == "") or args.only == "quantize":
         for i in range(10):
             quant_step(i)
         q_ms = _median_events_ms(quant_step, 50)
@@ -188,7 +188,7 @@ def main():
     del xsets
 
     # ---------------------------------------------------------------- decode sweep (cfg3)
-    if not args.no_extras or args.only == "decode":
+    if (not args.no_extras and args.only == "") or args.only == "decode":
         Nd = Kd = 8192
         wq3, ws3 = mslk_amd.quantize_fp8_row(W.cfg3_weight().to(dev))
         wsets = [wq3.clone() for _ in range(6)]  # 6 x 64 MiB > Infinity Cache

@@ -1,17 +1,24 @@
 // Skinny-M (decode) f8f8bf16_rowwise for gfx950: M <= 64, the weight matrix is streamed once.
 //
-// The op is HBM-bound: N*K weight bytes dominate (reference shape class: Llama-70B o_proj,
+// The op is HBM-bound: the N*K weight bytes dominate (reference shape class: Llama-70B o_proj;
 // csrc/gemm/ck/fp8_rowwise/fp8fp8bf16_rowwise_gemm.hip:422-468 sends M < 64 to a tiny-tile kernel).
-// Here every workgroup owns 16 weight rows (one MFMA n-fragment) and ALL of K:
-//   * the 4 wavefronts of the workgroup take the 128-byte K steps round-robin, so the workgroup
-//     reads 512 contiguous bytes of each of its rows per round;
-//   * weight fragments go global -> VGPR directly (each byte is used once: LDS would add nothing);
-//     lane (i = l & 15, g = l >> 4) loads bytes [16 g, 16 g + 16) and [64 + 16 g, 64 + 16 g + 16) of
-//     row i of the step, so one load instruction covers 64 contiguous bytes per row; the activation
-//     fragment uses the same k assignment (any shared permutation of k is a valid MFMA operand pair);
-//   * activations (M x K, a few hundred KB at most) are re-read from L2 by every workgroup;
-//   * the four per-wave partial sums meet in LDS; 256 lanes reduce, scale and store bf16.
-// There is no split-K across workgroups, hence no workspace and no atomics.
+// What matters is the number of bytes in flight per CU, so the kernel is organised around deep,
+// batched, register-resident loads and never touches LDS for the operands:
+//   * a workgroup of 8 wavefronts owns NT*16 weight rows and ALL of K; the wavefronts take the
+//     128-byte K steps round-robin (wave w: steps w, w+8, ...), so the workgroup reads 1 KiB of each of
+//     its rows per round and no cross-workgroup reduction (workspace, atomics) is needed;
+//   * per batch a wave issues the loads of U of its K steps (U * NT KiB * 2 of weights per wave) before
+//     the first MFMA consumes them;
+//   * weight fragments go global -> VGPR directly (each byte is used once).  Lane (i = l & 15, g = l >> 4)
+//     loads bytes [16 g, 16 g + 16) and [64 + 16 g, 64 + 16 g + 16) of row i of the step, so one load
+//     instruction covers 64 contiguous bytes per row; the activation fragment uses the same k
+//     assignment (any k permutation shared by both MFMA operands gives the same dot products);
+//   * activations (M x K, at most 512 KiB) are re-read from L2; each activation fragment is reused by
+//     the NT weight fragments of the step, which bounds the L2 traffic for M > 16;
+//   * the eight per-wave partial sums meet in LDS; the lanes reduce, scale and store bf16.
+#include <cstdio>
+#include <cstdlib>
+
 #include "common.h"
 #include "kernels.h"
 
@@ -22,79 +29,149 @@ constexpr int kStep = 128;
 
 MSLK_AMD_DEVINL v4i load16_or_zero(const uint8_t* p, bool ok) {
   v4i z = {0, 0, 0, 0};
-  return ok ? *reinterpret_cast<const v4i*>(p) : z;
+  if (ok) z = *reinterpret_cast<const v4i*>(p);
+  return z;
 }
 
-template <int MT, int BIAS>
-__global__ __launch_bounds__(256) void skinny_kernel(GemmProblem p) {
-  __shared__ float red[4][MT][256];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+// Weights are read exactly once: stream them past the caches.
+MSLK_AMD_DEVINL v4i load16_stream(const uint8_t* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+}
+
+// One batch: the loads of U K-steps of this wave (steps kt0, kt0 + 8, ...), then their MFMAs.
+// CHECKED = false is the fast path: every step lies fully inside K, so no lane is predicated.
+template <int MT, int NT, int U, int kWaves, bool CHECKED>
+MSLK_AMD_DEVINL void skinny_batch(const uint8_t* const (&wp)[NT], const uint8_t* const (&xp)[MT], int kt0, int K, int g,
+                                  v4f (&acc)[NT][MT]) {
+  v8i wf[U][NT], xf[U][MT];
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int k0 = (kt0 + u * kWaves) * kStep;
+    const bool ok0 = !CHECKED || k0 + g * 16 < K, ok1 = !CHECKED || k0 + 64 + g * 16 < K;
+#pragma unroll
+    for (int tn = 0; tn < NT; ++tn) {
+      v4i lo, hi;
+      if constexpr (CHECKED) {
+        lo = load16_or_zero(wp[tn] + k0, ok0);
+        hi = load16_or_zero(wp[tn] + k0 + 64, ok1);
+      } else {
+        lo = load16_stream(wp[tn] + k0);
+        hi = load16_stream(wp[tn] + k0 + 64);
+      }
+      wf[u][tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+#pragma unroll
+    for (int tm = 0; tm < MT; ++tm) {
+      v4i lo, hi;
+      if constexpr (CHECKED) {
+        lo = load16_or_zero(xp[tm] + k0, ok0);
+        hi = load16_or_zero(xp[tm] + k0 + 64, ok1);
+      } else {
+        lo = *reinterpret_cast<const v4i*>(xp[tm] + k0);
+        hi = *reinterpret_cast<const v4i*>(xp[tm] + k0 + 64);
+      }
+      xf[u][tm] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u)
+#pragma unroll
+    for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+      for (int tm = 0; tm < MT; ++tm)
+        acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[u][tn], xf[u][tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+}
+
+template <int MT, int NT, int U, int kWaves, int BIAS>
+__global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
+  __shared__ float red[kWaves][NT][MT][256];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int i = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16;
+  const int n0 = blockIdx.x * (NT * 16);
   const int K = p.K;
-  const int w_row = (n0 + i < p.N) ? n0 + i : p.N - 1;
-  const uint8_t* wp = p.wq + (int64_t)w_row * K + g * 16;
+
+  // Rows beyond N / M are clamped to the last valid row: an MFMA output row or column depends only on
+  // its own operand row, and the clamped ones are never stored.
+  const uint8_t* wp[NT];
+#pragma unroll
+  for (int tn = 0; tn < NT; ++tn) {
+    const int row = n0 + tn * 16 + i;
+    wp[tn] = p.wq + (int64_t)(row < p.N ? row : p.N - 1) * K + g * 16;
+  }
   const uint8_t* xp[MT];
-  bool xok[MT];
 #pragma unroll
   for (int tm = 0; tm < MT; ++tm) {
     const int m = tm * 16 + i;
-    xok[tm] = m < p.M;
-    xp[tm] = p.xq + (int64_t)(xok[tm] ? m : 0) * K + g * 16;
+    xp[tm] = p.xq + (int64_t)(m < p.M ? m : p.M - 1) * K + g * 16;
   }
-  v4f acc[MT];
+  v4f acc[NT][MT];
 #pragma unroll
-  for (int tm = 0; tm < MT; ++tm) acc[tm] = v4f{0.f, 0.f, 0.f, 0.f};
+  for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < MT; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // Epilogue operands are fetched before the weight stream so that their (cold) latency is hidden:
+  // value index t = 4 * l + r of a fragment holds D[n = 4 * (l >> 4) + r][m = l & 15]; the 512 lanes
+  // cover the NT * MT * 256 values in ROUNDS rounds.
+  constexpr int ROUNDS = (NT * MT * 256 + kWaves * 64 - 1) / (kWaves * 64);
+  float e_xs[ROUNDS], e_ws[ROUNDS], e_b[ROUNDS];
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int v = threadIdx.x + r * kWaves * 64;
+    const int frag = v >> 8, t = v & 255;
+    const int tn = frag / MT, tm = frag % MT;
+    const int n = n0 + tn * 16 + 4 * (t >> 6) + (t & 3);
+    const int m = tm * 16 + ((t >> 2) & 15);
+    const bool ok = frag < NT * MT && n < p.N && m < p.M;
+    e_xs[r] = ok ? p.xs[m] : 0.f;
+    e_ws[r] = ok ? p.ws[n] : 0.f;
+    e_b[r] = 0.f;
+    if constexpr (BIAS == 1) e_b[r] = ok ? reinterpret_cast<const float*>(p.bias)[n] : 0.f;
+    if constexpr (BIAS == 2) e_b[r] = ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]) : 0.f;
+  }
 
   const int KT = (K + kStep - 1) / kStep;
-#pragma unroll 4
-  for (int kt = wave; kt < KT; kt += 4) {
-    const int k0 = kt * kStep;
-    const bool ok0 = k0 + g * 16 < K, ok1 = k0 + 64 + g * 16 < K;
-    const v4i wlo = load16_or_zero(wp + k0, ok0);
-    const v4i whi = load16_or_zero(wp + k0 + 64, ok1);
-    const v8i wf = __builtin_shufflevector(wlo, whi, 0, 1, 2, 3, 4, 5, 6, 7);
-#pragma unroll
-    for (int tm = 0; tm < MT; ++tm) {
-      const v4i xlo = load16_or_zero(xp[tm] + k0, ok0 && xok[tm]);
-      const v4i xhi = load16_or_zero(xp[tm] + k0 + 64, ok1 && xok[tm]);
-      const v8i xf = __builtin_shufflevector(xlo, xhi, 0, 1, 2, 3, 4, 5, 6, 7);
-      acc[tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf, acc[tm], 0, 0, 0, 0, 0, 0);
-    }
+  int kt0 = wave;
+  if (K % (kWaves * kStep) == 0) {
+    // every wave owns the same number of complete steps: unpredicated batches
+    for (; kt0 + (U - 1) * kWaves < KT; kt0 += kWaves * U) skinny_batch<MT, NT, U, kWaves, false>(wp, xp, kt0, K, g, acc);
+    for (; kt0 < KT; kt0 += kWaves) skinny_batch<MT, NT, 1, kWaves, false>(wp, xp, kt0, K, g, acc);
+  } else {
+    for (; kt0 < KT; kt0 += kWaves * 2) skinny_batch<MT, NT, 2, kWaves, true>(wp, xp, kt0, K, g, acc);
   }
 
 #pragma unroll
-  for (int tm = 0; tm < MT; ++tm)
-    *reinterpret_cast<v4f*>(&red[wave][tm][lane * 4]) = acc[tm];
+  for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < MT; ++tm)
+      *reinterpret_cast<v4f*>(&red[wave][tn][tm][lane * 4]) = acc[tn][tm];
   __syncthreads();
 
-  // value index t = 4 * lane' + r holds D[n = 4 * (lane' >> 4) + r][m = lane' & 15]
-  const int t = threadIdx.x;
-  const int n = n0 + 4 * (t >> 6) + (t & 3);
-  const int mj = (t >> 2) & 15;
-  if (n >= p.N) return;
-  const float wsn = p.ws[n];
-  float bn = 0.f;
-  if constexpr (BIAS == 1) bn = reinterpret_cast<const float*>(p.bias)[n];
-  if constexpr (BIAS == 2) bn = bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]);
 #pragma unroll
-  for (int tm = 0; tm < MT; ++tm) {
-    const int m = tm * 16 + mj;
-    if (m >= p.M) continue;
-    const float sum = (red[0][tm][t] + red[1][tm][t]) + (red[2][tm][t] + red[3][tm][t]);
-    float v = (sum * p.xs[m]) * wsn;
-    if constexpr (BIAS != 0) v += bn;
-    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_bf16_bits(v);
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int v = threadIdx.x + r * kWaves * 64;
+    const int frag = v >> 8, t = v & 255;
+    const int tn = frag / MT, tm = frag % MT;
+    const int n = n0 + tn * 16 + 4 * (t >> 6) + (t & 3);
+    const int m = tm * 16 + ((t >> 2) & 15);
+    if (frag >= NT * MT || n >= p.N || m >= p.M) continue;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += red[w][tn][tm][t];
+    float val = (sum * e_xs[r]) * e_ws[r];
+    if constexpr (BIAS != 0) val += e_b[r];
+    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_bf16_bits(val);
   }
 }
 
-template <int MT>
-hipError_t launch_mt(const GemmProblem& p, hipStream_t s) {
-  const unsigned grid = (unsigned)((p.N + 15) / 16);
+template <int MT, int NT, int U, int kWaves = 8>
+hipError_t launch_cfg(const GemmProblem& p, hipStream_t s) {
+  const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
   switch (p.bias_dtype) {
-    case 0: skinny_kernel<MT, 0><<<grid, 256, 0, s>>>(p); break;
-    case 1: skinny_kernel<MT, 1><<<grid, 256, 0, s>>>(p); break;
-    default: skinny_kernel<MT, 2><<<grid, 256, 0, s>>>(p); break;
+    case 0: skinny_kernel<MT, NT, U, kWaves, 0><<<grid, kWaves * 64, 0, s>>>(p); break;
+    case 1: skinny_kernel<MT, NT, U, kWaves, 1><<<grid, kWaves * 64, 0, s>>>(p); break;
+    default: skinny_kernel<MT, NT, U, kWaves, 2><<<grid, kWaves * 64, 0, s>>>(p); break;
   }
   return hipGetLastError();
 }
@@ -108,10 +185,21 @@ bool skinny_supports(const GemmProblem& p) {
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
   if (!skinny_supports(p)) return hipErrorInvalidValue;
-  if (p.M <= 16) return launch_mt<1>(p, s);
-  if (p.M <= 32) return launch_mt<2>(p, s);
-  if (p.M <= 48) return launch_mt<3>(p, s);
-  return launch_mt<4>(p, s);
+#ifdef MSLK_EXP_SWEEP
+  if (const char* e = getenv("MSLK_SKINNY_CFG")) {
+    int mt = 0, nt = 0, u = 0, w = 0;
+    sscanf(e, "%d,%d,%d,%d", &mt, &nt, &u, &w);
+    if (mt * 16 < p.M) return hipErrorInvalidValue;
+#define TRY(MT_, NT_, U_, W_) if (mt == MT_ && nt == NT_ && u == U_ && w == W_) return launch_cfg<MT_, NT_, U_, W_>(p, s);
+    TRY(1,1,8,8) TRY(1,1,4,8) TRY(1,1,8,4) TRY(1,1,4,4) TRY(1,1,4,16) TRY(1,1,2,16) TRY(1,2,4,8) TRY(1,2,8,8) TRY(1,2,4,4) TRY(1,2,8,4)
+    TRY(4,1,2,8) TRY(4,1,4,8) TRY(4,2,2,8) TRY(4,2,4,8) TRY(4,1,2,4) TRY(4,1,4,4) TRY(4,2,2,4) TRY(4,2,4,4) TRY(4,1,2,16) TRY(4,4,2,8) TRY(4,4,2,4) TRY(4,4,1,8)
+    return hipErrorInvalidValue;
+  }
+#endif
+  if (p.M <= 16) return launch_cfg<1, 1, 8>(p, s);
+  if (p.M <= 32) return launch_cfg<2, 2, 4>(p, s);
+  if (p.M <= 48) return launch_cfg<3, 2, 4>(p, s);
+  return launch_cfg<4, 2, 4>(p, s);
 }
 
 }  // namespace mslk_amd
