@@ -48,6 +48,12 @@ MSLK_AMD_DEVINL void wait_vmcnt0() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
+// The output is written once and not re-read by this kernel: a streaming (non-temporal) store keeps
+// it from displacing the operand tiles in L2 and from piling up as dirty lines to flush at kernel end.
+MSLK_AMD_DEVINL void store16_stream(uint16_t* dst, uint4 val) {
+  __builtin_nontemporal_store(v4i{(int)val.x, (int)val.y, (int)val.z, (int)val.w}, reinterpret_cast<v4i*>(dst));
+}
+
 MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
 }
@@ -70,8 +76,18 @@ __device__ unsigned long long g_trace[4096];
 #define MSLK_TILE_TRACE_RT(slot) do {} while (0)
 #endif
 
+#ifdef MSLK_EXP_TRACE
+#define MSLK_STAMP(i) do { if (trace_on) tr[i] = __builtin_amdgcn_s_memtime(); } while (0)
+#else
+#define MSLK_STAMP(i) do {} while (0)
+#endif
+
 template <typename TS, int BIAS>
 struct GemmTile {
+#ifdef MSLK_EXP_TRACE
+  unsigned long long tr[8];
+  bool trace_on;
+#endif
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
   uint32_t b_off[TS::LB];
@@ -187,25 +203,40 @@ struct GemmTile {
     const FragOff fo = frag_off();
     const char* b_tile = b_tile_of(cur);
     v8i wf = wf0;
+    MSLK_STAMP(0);
 #pragma unroll
     for (int tn = 0; tn < TS::FN - 1; ++tn) {
-      const v8i wf_next = load_frag(b_tile, tn + 1, fo);
-      if constexpr (DMA) {
-        if (tn < HALF) {
+      if (tn == HALF) MSLK_STAMP(1);
+      // Issue order inside a group: the read of the next WQ fragment follows the first MFMA, the DMA
+      // loads follow the last MFMAs, one each.  Every DMA sits in the shadow of an MFMA, and the
+      // LDS reads issued before it are at least four MFMAs old: the compiler orders all earlier LDS
+      // reads before a DMA write (it cannot see that the two stages are disjoint), so a DMA right
+      // behind a fresh read would stall on that read's latency.
+      constexpr int NDMA = PA + PB;
+      static_assert(NDMA <= TS::FM, "one DMA per MFMA slot");
+      v8i wf_next;
 #pragma unroll
-          for (int u = 0; u < PA; ++u) issue_a(nxt, k_next, tn * PA + u);
-#pragma unroll
-          for (int u = 0; u < PB; ++u) issue_b(nxt, k_next, tn * PB + u);
-        }
-      }
-#pragma unroll
-      for (int tm = 0; tm < TS::FM; ++tm)
+      for (int tm = 0; tm < TS::FM; ++tm) {
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+        if (tm == 0) wf_next = load_frag(b_tile, tn + 1, fo);
+        if constexpr (DMA) {
+          const int d = tm - (TS::FM - NDMA);
+          if (tn < HALF && d >= 0) {
+            if (d < PA) issue_a(nxt, k_next, tn * PA + d);
+            else issue_b(nxt, k_next, tn * PB + (d - PA));
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
       wf = wf_next;
       __builtin_amdgcn_sched_barrier(0);
     }
+    MSLK_STAMP(2);
     if constexpr (NEXT) {
+      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+      MSLK_STAMP(3);
       __syncthreads();  // s_waitcnt vmcnt(0) lgkmcnt(0); s_barrier
+      MSLK_STAMP(4);
       wf0 = load_frag(b_tile_of(nxt), 0, fo);
     }
     const char* a_next = a_tile_of(nxt);
@@ -218,6 +249,7 @@ struct GemmTile {
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+    MSLK_STAMP(5);
   }
 
   // Whole tile: K loop + epilogue.  m_rem / n_rem = valid rows / columns of this tile (>= 1).
@@ -244,6 +276,9 @@ struct GemmTile {
       load_first_frags(cur, xf, wf0);
       for (int kt = 0; kt < KT - 1; ++kt) {
         MSLK_TILE_TRACE(kt * 4 + 0);
+#ifdef MSLK_EXP_TRACE
+        trace_on = (kt == 12);
+#endif
         step<true, true>(cur, nxt, (kt + 1) * kBK, acc, xf, wf0);
         char* t = cur; cur = nxt; nxt = t;
       }
@@ -262,6 +297,9 @@ struct GemmTile {
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
     MSLK_TILE_TRACE(32 * 4 + 1);
     MSLK_TILE_TRACE_RT(142);
+#ifdef MSLK_EXP_TRACE
+    if (threadIdx.x == 0 && blockIdx.x == 0) for (int q = 0; q < 6; ++q) g_trace[200 + q] = tr[q];
+#endif
   }
 
   // Epilogue.  A lane's accumulators of one 16-row m fragment are 4 consecutive n in each of the
@@ -272,6 +310,15 @@ struct GemmTile {
   // BN/2 bf16 (16 lanes x 16 bytes each).
   MSLK_AMD_DEVINL void epilogue(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                 const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
+    // Interior tiles (the common case) take a path without any per-element bounds logic.
+    const bool full = m_rem >= TS::kBM && n_rem >= TS::kBN && (N & 7) == 0;
+    if (full) epilogue_impl<true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+    else epilogue_impl<false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+  }
+
+  template <bool FULL>
+  MSLK_AMD_DEVINL void epilogue_impl(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
+                                     const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     constexpr int WN = TS::kBN / 2;              // columns per wave
     constexpr int PITCH = WN * 2 + 16;           // bytes per staged row
     constexpr int BUF = 16 * PITCH;
@@ -287,23 +334,39 @@ struct GemmTile {
 
     float wsv[TS::FN][4], bv[TS::FN][4];
 #pragma unroll
-    for (int tn = 0; tn < TS::FN; ++tn)
+    for (int tn = 0; tn < TS::FN; ++tn) {
+      const int n = n_base + tn * 16 + 4 * q;
+      if constexpr (FULL) {
+        const float4 w4 = *reinterpret_cast<const float4*>(ws + n);
+        wsv[tn][0] = w4.x; wsv[tn][1] = w4.y; wsv[tn][2] = w4.z; wsv[tn][3] = w4.w;
+        if constexpr (BIAS == 1) {
+          const float4 b4 = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(bias) + n);
+          bv[tn][0] = b4.x; bv[tn][1] = b4.y; bv[tn][2] = b4.z; bv[tn][3] = b4.w;
+        } else if constexpr (BIAS == 2) {
+          const uint2 b2 = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(bias) + n);
+          bv[tn][0] = bf16_bits_to_f32(b2.x & 0xFFFFu); bv[tn][1] = bf16_bits_to_f32(b2.x >> 16);
+          bv[tn][2] = bf16_bits_to_f32(b2.y & 0xFFFFu); bv[tn][3] = bf16_bits_to_f32(b2.y >> 16);
+        } else {
+          bv[tn][0] = bv[tn][1] = bv[tn][2] = bv[tn][3] = 0.f;
+        }
+      } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int n = n_base + tn * 16 + 4 * q + r;
-        const bool ok = n < n_rem;
-        wsv[tn][r] = ok ? ws[n] : 0.f;
-        if constexpr (BIAS == 1) bv[tn][r] = ok ? reinterpret_cast<const float*>(bias)[n] : 0.f;
-        else if constexpr (BIAS == 2) bv[tn][r] = ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(bias)[n]) : 0.f;
-        else bv[tn][r] = 0.f;
+        for (int r = 0; r < 4; ++r) {
+          const bool ok = n + r < n_rem;
+          wsv[tn][r] = ok ? ws[n + r] : 0.f;
+          if constexpr (BIAS == 1) bv[tn][r] = ok ? reinterpret_cast<const float*>(bias)[n + r] : 0.f;
+          else if constexpr (BIAS == 2) bv[tn][r] = ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(bias)[n + r]) : 0.f;
+          else bv[tn][r] = 0.f;
+        }
       }
+    }
 
     const int rd_row = lane / CH, rd_chunk = lane % CH;
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
       char* b = buf + (tm & 1) * BUF;
       const int m = m_base + tm * 16 + j;
-      const float xsv = m < m_rem ? xs[m] : 0.f;
+      const float xsv = (FULL || m < m_rem) ? xs[m] : 0.f;
 #pragma unroll
       for (int tn = 0; tn < TS::FN; ++tn) {
         float v[4];
@@ -324,15 +387,19 @@ struct GemmTile {
         const uint4 val = *reinterpret_cast<const uint4*>(b + row * PITCH + rd_chunk * 16);
         const int mm = m_base + tm * 16 + row;
         const int nn = n_base + rd_chunk * 8;
-        if (mm >= m_rem || nn >= n_rem) continue;
         uint16_t* dst = y + (int64_t)mm * N + nn;
-        if (vec_store && nn + 7 < n_rem) {
-          *reinterpret_cast<uint4*>(dst) = val;
+        if constexpr (FULL) {
+          store16_stream(dst, val);
         } else {
-          const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+          if (mm >= m_rem || nn >= n_rem) continue;
+          if (vec_store && nn + 7 < n_rem) {
+            store16_stream(dst, val);
+          } else {
+            const uint32_t w[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            if (nn + e < n_rem) dst[e] = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
+            for (int e = 0; e < 8; ++e)
+              if (nn + e < n_rem) dst[e] = (uint16_t)(w[e >> 1] >> ((e & 1) * 16));
+          }
         }
       }
     }
