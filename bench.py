@@ -29,6 +29,19 @@ PEAK_FP8_FLOPS_REF = 4.6e15  # the figure the reference's bench uses for gfx950 
 PEAK_HBM_BPS = 8.0e12
 
 
+def _measured_traffic_bytes():
+    """HBM-side bytes per 4096^3 GEMM launch from the committed rocprofv3 FETCH_SIZE/WRITE_SIZE summary
+    (counters cannot be read from inside this process); None when the summary is absent."""
+    path = os.path.join(ROOT, "profiles", "gemm_4096_traffic_pmc.txt")
+    try:
+        for ln in open(path):
+            if ln.startswith("traffic per launch ="):
+                return float(ln.split("=")[1].split("MB")[0]) * 1e6
+    except OSError:
+        pass
+    return None
+
+
 def _events_ms(fn, iters):
     """Average duration of fn() in ms, HIP events on the current stream (the one kernels launch on)."""
     import torch
@@ -64,6 +77,17 @@ class CApi:
         self.check(self.L.mslk_amd_f8f8bf16_rowwise(xq.data_ptr(), wq.data_ptr(), xs.data_ptr(), ws.data_ptr(),
                                                     None if bias is None else bias.data_ptr(), bcode, y.data_ptr(),
                                                     M, N, K, None, 0, self.stream))
+
+    def grouped_call(self, xq, wq, xs, ws, ys):
+        """Pre-marshalled TensorList call: returns a closure that only crosses the C ABI."""
+        import ctypes
+        G = len(xq)
+        P = ctypes.c_void_p * G
+        I = ctypes.c_int64 * G
+        args = (G, P(*[t.data_ptr() for t in xq]), P(*[t.data_ptr() for t in wq]), P(*[t.data_ptr() for t in xs]),
+                P(*[t.data_ptr() for t in ws]), P(*[t.data_ptr() for t in ys]), I(*[t.shape[0] for t in xq]),
+                I(*[t.shape[0] for t in wq]), I(*[t.shape[1] for t in wq]), self.stream)
+        return lambda: self.check(self.L.mslk_amd_f8f8bf16_rowwise_grouped(*args))
 
     def quantize(self, x, xq, scale):
         rows, K = x.shape
@@ -106,7 +130,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", default="", help="profile helper: run only this piece (gemm|quantize|decode) and exit")
+    ap.add_argument("--only", default="", help="profile helper: run only this piece (gemm|quantize|decode|traffic) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -138,6 +162,18 @@ def main():
         api.gemm(xq, wq, xs, ws, y)
 
     flops = 2.0 * M * N * K
+    if args.only == "traffic":
+        # Counter calibration for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`: a plain device copy of known
+        # size (256 MiB read + 256 MiB written by one elementwise kernel) next to a few GEMM launches.
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        for i in range(12):
+            gemm_step(i)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_each_way": 256 << 20, "gemm_launches": 12}))
+        return
     if args.only in ("", "gemm"):
         for i in range(args.warmup):
             gemm_step(i)
@@ -248,9 +284,11 @@ def main():
             wq4.append(q)
             ws4.append(s)
         xl, sl = list(xq4.split(wl4.counts)), list(xs4.split(wl4.counts))
+        ys4 = torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4)
+        call4 = api.grouped_call(xl, wq4, sl, ws4, ys4)
         for _ in range(3):
-            torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4)
-        ms = _median_events_ms(lambda i: torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4), 10)
+            call4()
+        ms = _median_events_ms(lambda i: call4(), 10)
         f4 = 2.0 * 8192 * 8192 * 5120
         extras["grouped_cfg4_16x8192x5120"] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12,
                                                 "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS, "counts": wl4.counts}
@@ -273,7 +311,7 @@ def main():
         "pct_of_reference_peak_4.6PF": 100.0 * value * 1e12 / PEAK_FP8_FLOPS_REF,
         "roofline": {"kernel": "dense_tiled_kernel<256,256> (f8f8bf16_rowwise 4096^3)", "bound": "mfma",
                      "achieved": achieved, "peak": PEAK_FP8_FLOPS / 1e12, "unit": "TFLOP/s",
-                     "frac": achieved * 1e12 / PEAK_FP8_FLOPS, "traffic": None, "kernel_ms": kern_ms,
+                     "frac": achieved * 1e12 / PEAK_FP8_FLOPS, "traffic": _measured_traffic_bytes(), "kernel_ms": kern_ms,
                      "flops_per_launch": flops},
         "cpu_baseline": cpu,
         "extras": extras,

@@ -51,15 +51,22 @@ template <> struct Traits<2> {  // fp32
 template <int DTYPE> struct Vec8 { uint4 w; };          // 8 x 16-bit
 template <> struct Vec8<2> { uint4 lo, hi; };           // 8 x fp32
 
+MSLK_AMD_DEVINL void store8_stream(uint2* dst, uint2 val) {
+  __builtin_nontemporal_store(v2i{(int)val.x, (int)val.y}, reinterpret_cast<v2i*>(dst));
+}
+
 template <int DTYPE>
 MSLK_AMD_DEVINL Vec8<DTYPE> load_vec8(const void* row_ptr, int vec_idx) {
   Vec8<DTYPE> v;
+  // the input is read once (rows cached in registers) or twice in quick succession: stream it
   if constexpr (DTYPE == 2) {
-    const uint4* p = reinterpret_cast<const uint4*>(row_ptr) + 2 * (int64_t)vec_idx;
-    v.lo = p[0];
-    v.hi = p[1];
+    const v4i* p = reinterpret_cast<const v4i*>(row_ptr) + 2 * (int64_t)vec_idx;
+    const v4i a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
+    v.lo = make_uint4(a.x, a.y, a.z, a.w);
+    v.hi = make_uint4(b.x, b.y, b.z, b.w);
   } else {
-    v.w = reinterpret_cast<const uint4*>(row_ptr)[vec_idx];
+    const v4i a = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(row_ptr) + vec_idx);
+    v.w = make_uint4(a.x, a.y, a.z, a.w);
   }
   return v;
 }
@@ -186,11 +193,11 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = i * TEAM + lane;
-      if (idx < nvec) out_row[idx] = quantize_vec8<DTYPE>(cache[i], inv);
+      if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE>(cache[i], inv));
     }
   } else {
     for (int idx = lane; idx < nvec; idx += TEAM)
-      out_row[idx] = quantize_vec8<DTYPE>(load_vec8<DTYPE>(row_ptr, idx), inv);
+      store8_stream(out_row + idx, quantize_vec8<DTYPE>(load_vec8<DTYPE>(row_ptr, idx), inv));
   }
   // zero padding columns [K, out_stride)
   for (int64_t k = K + lane; k < out_stride; k += TEAM) out[row * out_stride + k] = 0;
