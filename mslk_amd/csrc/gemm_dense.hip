@@ -102,9 +102,4 @@ hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s) {
   return hipGetLastError();
 }
 
-#ifdef MSLK_EXP_TRACE
-extern "C" int mslk_exp_read_trace(unsigned long long* out, int n) {
-  return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(g_trace), n * sizeof(unsigned long long));
-}
-#endif
 }  // namespace mslk_amd

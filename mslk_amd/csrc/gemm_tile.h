@@ -58,36 +58,9 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
   __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
 }
 
-#ifdef MSLK_EXP_TRACE
-__device__ unsigned long long g_trace[4096];
-#define MSLK_TILE_TRACE(slot)                                                            \
-  do {                                                                                   \
-    if (threadIdx.x == 0 && blockIdx.x == 0 && (slot) < 4096) g_trace[slot] = __builtin_amdgcn_s_memtime(); \
-  } while (0)
-#else
-#define MSLK_TILE_TRACE(slot) do {} while (0)
-#endif
-#ifdef MSLK_EXP_TRACE
-#define MSLK_TILE_TRACE_RT(slot)                                                         \
-  do {                                                                                   \
-    if (threadIdx.x == 0 && blockIdx.x == 0) g_trace[slot] = __builtin_amdgcn_s_memrealtime(); \
-  } while (0)
-#else
-#define MSLK_TILE_TRACE_RT(slot) do {} while (0)
-#endif
-
-#ifdef MSLK_EXP_TRACE
-#define MSLK_STAMP(i) do { if (trace_on) tr[i] = __builtin_amdgcn_s_memtime(); } while (0)
-#else
-#define MSLK_STAMP(i) do {} while (0)
-#endif
 
 template <typename TS, int BIAS>
 struct GemmTile {
-#ifdef MSLK_EXP_TRACE
-  unsigned long long tr[8];
-  bool trace_on;
-#endif
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
   uint32_t b_off[TS::LB];
@@ -203,10 +176,8 @@ struct GemmTile {
     const FragOff fo = frag_off();
     const char* b_tile = b_tile_of(cur);
     v8i wf = wf0;
-    MSLK_STAMP(0);
 #pragma unroll
     for (int tn = 0; tn < TS::FN - 1; ++tn) {
-      if (tn == HALF) MSLK_STAMP(1);
       // Issue order inside a group: the read of the next WQ fragment follows the first MFMA, the DMA
       // loads follow the last MFMAs, one each.  Every DMA sits in the shadow of an MFMA, and the
       // LDS reads issued before it are at least four MFMAs old: the compiler orders all earlier LDS
@@ -231,12 +202,8 @@ struct GemmTile {
       wf = wf_next;
       __builtin_amdgcn_sched_barrier(0);
     }
-    MSLK_STAMP(2);
     if constexpr (NEXT) {
-      __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
-      MSLK_STAMP(3);
       __syncthreads();  // s_waitcnt vmcnt(0) lgkmcnt(0); s_barrier
-      MSLK_STAMP(4);
       wf0 = load_frag(b_tile_of(nxt), 0, fo);
     }
     const char* a_next = a_tile_of(nxt);
@@ -249,15 +216,12 @@ struct GemmTile {
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    MSLK_STAMP(5);
   }
 
   // Whole tile: K loop + epilogue.  m_rem / n_rem = valid rows / columns of this tile (>= 1).
   // xq_tile / wq_tile / xs / ws / bias / y are already offset to the tile's first row and column.
   MSLK_AMD_DEVINL void run(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, const float* xs,
                            const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K) {
-    MSLK_TILE_TRACE(140);
-    MSLK_TILE_TRACE_RT(141);
     init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, K);
     v4f acc[TS::FN][TS::FM];
 #pragma unroll
@@ -275,10 +239,6 @@ struct GemmTile {
       __syncthreads();
       load_first_frags(cur, xf, wf0);
       for (int kt = 0; kt < KT - 1; ++kt) {
-        MSLK_TILE_TRACE(kt * 4 + 0);
-#ifdef MSLK_EXP_TRACE
-        trace_on = (kt == 12);
-#endif
         step<true, true>(cur, nxt, (kt + 1) * kBK, acc, xf, wf0);
         char* t = cur; cur = nxt; nxt = t;
       }
@@ -292,14 +252,8 @@ struct GemmTile {
       load_first_frags(cur, xf, wf0);
       step<false, false>(cur, nxt, 0, acc, xf, wf0);
     }
-    MSLK_TILE_TRACE(32 * 4 + 0);
     __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
-    MSLK_TILE_TRACE(32 * 4 + 1);
-    MSLK_TILE_TRACE_RT(142);
-#ifdef MSLK_EXP_TRACE
-    if (threadIdx.x == 0 && blockIdx.x == 0) for (int q = 0; q < 6; ++q) g_trace[200 + q] = tr[q];
-#endif
   }
 
   // Epilogue.  A lane's accumulators of one 16-row m fragment are 4 consecutive n in each of the
@@ -310,12 +264,14 @@ struct GemmTile {
   // BN/2 bf16 (16 lanes x 16 bytes each).
   MSLK_AMD_DEVINL void epilogue(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                 const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
-    // Interior tiles (the common case) take a path without any per-element bounds logic.
-    const bool full = m_rem >= TS::kBM && n_rem >= TS::kBN && (N & 7) == 0;
+    // Tiles whose columns are all valid (the common case, also for the ragged last row tile of an MoE
+    // group) take a path whose only bounds logic is one row test per store instruction.
+    const bool full = n_rem >= TS::kBN && (N & 7) == 0;
     if (full) epilogue_impl<true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
     else epilogue_impl<false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
   }
 
+  // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged.
   template <bool FULL>
   MSLK_AMD_DEVINL void epilogue_impl(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                      const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
@@ -366,7 +322,7 @@ struct GemmTile {
     for (int tm = 0; tm < TS::FM; ++tm) {
       char* b = buf + (tm & 1) * BUF;
       const int m = m_base + tm * 16 + j;
-      const float xsv = (FULL || m < m_rem) ? xs[m] : 0.f;
+      const float xsv = m < m_rem ? xs[m] : 0.f;
 #pragma unroll
       for (int tn = 0; tn < TS::FN; ++tn) {
         float v[4];
@@ -389,7 +345,7 @@ struct GemmTile {
         const int nn = n_base + rd_chunk * 8;
         uint16_t* dst = y + (int64_t)mm * N + nn;
         if constexpr (FULL) {
-          store16_stream(dst, val);
+          if (mm < m_rem) store16_stream(dst, val);
         } else {
           if (mm >= m_rem || nn >= n_rem) continue;
           if (vec_store && nn + 7 < n_rem) {
