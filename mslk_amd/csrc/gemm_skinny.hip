@@ -16,9 +16,6 @@
 //   * activations (M x K, at most 512 KiB) are re-read from L2; each activation fragment is reused by
 //     the NT weight fragments of the step, which bounds the L2 traffic for M > 16;
 //   * the eight per-wave partial sums meet in LDS; the lanes reduce, scale and store bf16.
-#include <cstdio>
-#include <cstdlib>
-
 #include "common.h"
 #include "kernels.h"
 
@@ -176,6 +173,164 @@ hipError_t launch_cfg(const GemmProblem& p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Variant for 4 < M <= 64: activations staged through LDS.
+//
+// With more than a few activation rows the direct activation loads above become the bottleneck: one
+// load instruction then touches 16 different 128-byte lines (64 bytes of each), and the texture path
+// handles such an instruction four times slower than one that covers 8 full lines.  Here every wave
+// copies the activation rows of its own K steps global -> LDS with DMA loads of 8 full lines each
+// (the same XOR-swizzled 128-byte rows as the tiled kernel) and reads its MFMA fragments back from
+// LDS; the buffer is private to the wave, so no barrier is involved.  Weights still stream straight
+// into registers.  Requires K % (8 * 128) == 0.
+// ---------------------------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
+
+MSLK_AMD_DEVINL int row_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
+
+template <int MT, int NT, int U, int BIAS>
+__global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
+  constexpr int kWaves = 8;
+  constexpr int XBUF = U * MT * 2048;                       // bytes of staged activations per wave
+  static_assert(XBUF >= NT * MT * 1024, "the reduction slot of a wave lives inside its staging buffer");
+  __shared__ __attribute__((aligned(1024))) char lds[kWaves * XBUF];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * (NT * 16);
+  const int K = p.K;
+  char* xbuf = lds + wave * XBUF;
+
+  const uint8_t* wp[NT];
+#pragma unroll
+  for (int tn = 0; tn < NT; ++tn) {
+    const int row = n0 + tn * 16 + i;
+    wp[tn] = p.wq + (int64_t)(row < p.N ? row : p.N - 1) * K + g * 16;
+  }
+  // DMA source offsets: load h (0 / 1) of m-tile tm covers rows tm*16 + 8h + (lane >> 3); lane fetches the
+  // logical 16-byte chunk that belongs at physical position (lane & 7) of its swizzled LDS row.
+  uint32_t x_off[MT][2];
+#pragma unroll
+  for (int tm = 0; tm < MT; ++tm)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = 8 * h + (lane >> 3);
+      const int m = tm * 16 + r;
+      x_off[tm][h] = (uint32_t)(m < p.M ? m : p.M - 1) * (uint32_t)K + (((lane & 7) ^ row_swz(r)) << 4);
+    }
+  // Fragment read offsets: lane (i, g) reads logical chunks g and g + 4 of row i (the k assignment of the
+  // weight fragments above).
+  const int xr0 = i * 128 + ((g ^ row_swz(i)) << 4);
+  const int xr1 = i * 128 + (((g + 4) ^ row_swz(i)) << 4);
+
+  v4f acc[NT][MT];
+#pragma unroll
+  for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < MT; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  constexpr int ROUNDS = (NT * MT * 256 + kWaves * 64 - 1) / (kWaves * 64);
+  float e_xs[ROUNDS], e_ws[ROUNDS], e_b[ROUNDS];
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int v = threadIdx.x + r * kWaves * 64;
+    const int frag = v >> 8, t = v & 255;
+    const int tn = frag / MT, tm = frag % MT;
+    const int n = n0 + tn * 16 + 4 * (t >> 6) + (t & 3);
+    const int m = tm * 16 + ((t >> 2) & 15);
+    const bool ok = frag < NT * MT && n < p.N && m < p.M;
+    e_xs[r] = ok ? p.xs[m] : 0.f;
+    e_ws[r] = ok ? p.ws[n] : 0.f;
+    e_b[r] = 0.f;
+    if constexpr (BIAS == 1) e_b[r] = ok ? reinterpret_cast<const float*>(p.bias)[n] : 0.f;
+    if constexpr (BIAS == 2) e_b[r] = ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]) : 0.f;
+  }
+
+  const int KT = K / kStep;   // K % (8 * 128) == 0: every wave owns KT / 8 complete steps
+  for (int kt0 = wave; kt0 < KT; kt0 += kWaves * U) {
+    v8i wf[U][NT];
+    // Weights first: their HBM requests must not queue behind the (L2-resident) activation traffic.
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = kt0 + u * kWaves;
+      if (kt < KT) {           // wave-uniform
+        const int k0 = kt * kStep;
+#pragma unroll
+        for (int tn = 0; tn < NT; ++tn) {
+          const v4i lo = load16_stream(wp[tn] + k0);
+          const v4i hi = load16_stream(wp[tn] + k0 + 64);
+          wf[u][tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = kt0 + u * kWaves;
+      if (kt < KT) {
+        const int k0 = kt * kStep;
+#pragma unroll
+        for (int tm = 0; tm < MT; ++tm)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(p.xq + k0 + x_off[tm][h]),
+                                             (lds_ptr_t)(xbuf + ((u * MT + tm) * 2 + h) * 1024), 16, 0, 0);
+      }
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMA has landed in its private buffer
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (kt0 + u * kWaves < KT) {
+#pragma unroll
+        for (int tm = 0; tm < MT; ++tm) {
+          const char* xt = xbuf + (u * MT + tm) * 2048;
+          const v4i lo = *reinterpret_cast<const v4i*>(xt + xr0);
+          const v4i hi = *reinterpret_cast<const v4i*>(xt + xr1);
+          const v8i xf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+          for (int tn = 0; tn < NT; ++tn)
+            acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[u][tn], xf, acc[tn][tm], 0, 0, 0, 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // Reduction across the 8 waves: each wave parks its partial tiles in its own (now dead) staging buffer.
+  float* red = reinterpret_cast<float*>(xbuf);
+#pragma unroll
+  for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+    for (int tm = 0; tm < MT; ++tm)
+      *reinterpret_cast<v4f*>(&red[(tn * MT + tm) * 256 + lane * 4]) = acc[tn][tm];
+  __syncthreads();
+#pragma unroll
+  for (int r = 0; r < ROUNDS; ++r) {
+    const int v = threadIdx.x + r * kWaves * 64;
+    const int frag = v >> 8, t = v & 255;
+    const int tn = frag / MT, tm = frag % MT;
+    const int n = n0 + tn * 16 + 4 * (t >> 6) + (t & 3);
+    const int m = tm * 16 + ((t >> 2) & 15);
+    if (frag >= NT * MT || n >= p.N || m >= p.M) continue;
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += reinterpret_cast<const float*>(lds + w * XBUF)[frag * 256 + t];
+    float val = (sum * e_xs[r]) * e_ws[r];
+    if constexpr (BIAS != 0) val += e_b[r];
+    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_bf16_bits(val);
+  }
+}
+
+template <int MT, int NT, int U>
+hipError_t launch_xlds(const GemmProblem& p, hipStream_t s) {
+  const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
+  switch (p.bias_dtype) {
+    case 0: skinny_xlds_kernel<MT, NT, U, 0><<<grid, 512, 0, s>>>(p); break;
+    case 1: skinny_xlds_kernel<MT, NT, U, 1><<<grid, 512, 0, s>>>(p); break;
+    default: skinny_xlds_kernel<MT, NT, U, 2><<<grid, 512, 0, s>>>(p); break;
+  }
+  return hipGetLastError();
+}
+
 }  // namespace
 
 bool skinny_supports(const GemmProblem& p) {
@@ -185,17 +340,11 @@ bool skinny_supports(const GemmProblem& p) {
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
   if (!skinny_supports(p)) return hipErrorInvalidValue;
-#ifdef MSLK_EXP_SWEEP
-  if (const char* e = getenv("MSLK_SKINNY_CFG")) {
-    int mt = 0, nt = 0, u = 0, w = 0;
-    sscanf(e, "%d,%d,%d,%d", &mt, &nt, &u, &w);
-    if (mt * 16 < p.M) return hipErrorInvalidValue;
-#define TRY(MT_, NT_, U_, W_) if (mt == MT_ && nt == NT_ && u == U_ && w == W_) return launch_cfg<MT_, NT_, U_, W_>(p, s);
-    TRY(1,1,8,8) TRY(1,1,4,8) TRY(1,1,8,4) TRY(1,1,4,4) TRY(1,1,4,16) TRY(1,1,2,16) TRY(1,2,4,8) TRY(1,2,8,8) TRY(1,2,4,4) TRY(1,2,8,4)
-    TRY(4,1,2,8) TRY(4,1,4,8) TRY(4,2,2,8) TRY(4,2,4,8) TRY(4,1,2,4) TRY(4,1,4,4) TRY(4,2,2,4) TRY(4,2,4,4) TRY(4,1,2,16) TRY(4,4,2,8) TRY(4,4,2,4) TRY(4,4,1,8)
-    return hipErrorInvalidValue;
+  if (p.M > 4 && p.K % (8 * kStep) == 0) {   // activations through LDS
+    if (p.M <= 16) return launch_xlds<1, 1, 4>(p, s);
+    if (p.M <= 32) return launch_xlds<2, 1, 4>(p, s);
+    return launch_xlds<4, 2, 2>(p, s);
   }
-#endif
   if (p.M <= 16) return launch_cfg<1, 1, 8>(p, s);
   if (p.M <= 32) return launch_cfg<2, 2, 4>(p, s);
   if (p.M <= 48) return launch_cfg<3, 2, 4>(p, s);
