@@ -38,6 +38,23 @@ def _stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+class _on_device:
+    """`with torch.cuda.device(d)` only when d is not already current (the switch costs microseconds)."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device: torch.device):
+        self.ctx = None if device.index in (None, torch.cuda.current_device()) else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+
+
 def _check(cond: bool, msg: str = "") -> None:
     if not cond:
         raise RuntimeError(msg or "Expected condition to be true (mslk_amd argument check)")
@@ -89,7 +106,7 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None):
     xs = x_scale.contiguous()
     ws = w_scale.contiguous()
     bias_ptr, bias_code, _keep = _bias_args(bias, N, XQ.device)
-    with torch.cuda.device(XQ.device):
+    with _on_device(XQ.device):
         _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise(
             XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
             M, N, K, None, 0, _stream_ptr(XQ.device)))
@@ -133,7 +150,7 @@ def _launch_grouped(XQ, WQ, x_scale, w_scale, outs: List[torch.Tensor]) -> None:
     PtrArr = ctypes.c_void_p * G
     I64Arr = ctypes.c_int64 * G
     dev = XQ[0].device
-    with torch.cuda.device(dev):
+    with _on_device(dev):
         _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped(
             G, PtrArr(*[t.data_ptr() for t in XQ]), PtrArr(*[t.data_ptr() for t in WQ]),
             PtrArr(*[t.data_ptr() for t in xs]), PtrArr(*[t.data_ptr() for t in ws]),
@@ -187,7 +204,7 @@ def f8f8bf16_rowwise_grouped_stacked(XQ, WQ, x_scale, w_scale, M_sizes) -> torch
     if K == 0:
         return Y.zero_()
     xs, ws, ms = x_scale.contiguous(), w_scale.contiguous(), M_sizes.contiguous()
-    with torch.cuda.device(XQ.device):
+    with _on_device(XQ.device):
         _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped_stacked(
             XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), ms.data_ptr(), G, total_M, N, K,
             Y.data_ptr(), _stream_ptr(XQ.device)))

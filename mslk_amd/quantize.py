@@ -20,7 +20,24 @@ def _stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor], align_rows_to: Optional[int]
+class _on_device:
+    """`with torch.cuda.device(d)` only when d is not already current (the switch costs microseconds)."""
+
+    __slots__ = ("ctx",)
+
+    def __init__(self, device: torch.device):
+        self.ctx = None if device.index in (None, torch.cuda.current_device()) else torch.cuda.device(device)
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+
+
+def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, align_rows_to: Optional[int] = None
                    ) -> Tuple[torch.Tensor, torch.Tensor]:
     if a.dtype not in _DTYPE_CODE:
         raise RuntimeError(f"quantize_fp8_row: unsupported input dtype {a.dtype} (bf16, fp16, fp32 are supported)")
@@ -53,20 +70,13 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor], align_rows
         scale_ub = scale_ub.to(device=a.device, dtype=torch.float32).reshape(-1)[:1].contiguous()
         ub_ptr = scale_ub.data_ptr()
     if rows > 0:
-        with torch.cuda.device(a.device):
+        with _on_device(a.device):
             _lib.check(_lib.lib().mslk_amd_quantize_fp8_row(
                 a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
                 scale.data_ptr(), ub_ptr, _stream_ptr(a.device)))
     return xq, scale
 
 
-@torch.library.custom_op("mslk::quantize_fp8_row", mutates_args=(), device_types="cuda")
-def _quantize_fp8_row_op(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None,
-                         align_rows_to: Optional[int] = None) -> Tuple[torch.Tensor, torch.Tensor]:
-    return _quantize_impl(a, scale_ub, align_rows_to)
-
-
-@_quantize_fp8_row_op.register_fake
 def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None):
     # shape function of the reference (fp8_quantize.py:381-407)
     K = a.shape[-1]
@@ -74,6 +84,14 @@ def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None):
         K = (K + align_rows_to - 1) // align_rows_to * align_rows_to
     return (torch.empty(tuple(a.shape[:-1]) + (K,), dtype=FP8_DTYPE, device=a.device),
             torch.empty(a.shape[:-1], dtype=torch.float32, device=a.device))
+
+
+# Registered with the low-level library API (a few microseconds of dispatch per call); GPU kernel only.
+_library = torch.library.Library("mslk", "FRAGMENT")
+if not hasattr(torch.ops.mslk, "quantize_fp8_row"):
+    _library.define("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, int? align_rows_to=None) -> (Tensor, Tensor)")
+    _library.impl("quantize_fp8_row", _quantize_impl, "CUDA")
+    torch.library.register_fake("mslk::quantize_fp8_row", _quantize_fp8_row_fake, lib=_library)
 
 
 def quantize_fp8_row(
