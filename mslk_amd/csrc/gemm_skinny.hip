@@ -174,15 +174,15 @@ hipError_t launch_cfg(const GemmProblem& p, hipStream_t s) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Variant for 4 < M <= 64: activations staged through LDS.
+// Main variant (K % 1024 == 0): both operands staged through wave-private LDS.
 //
-// With more than a few activation rows the direct activation loads above become the bottleneck: one
-// load instruction then touches 16 different 128-byte lines (64 bytes of each), and the texture path
-// handles such an instruction four times slower than one that covers 8 full lines.  Here every wave
-// copies the activation rows of its own K steps global -> LDS with DMA loads of 8 full lines each
-// (the same XOR-swizzled 128-byte rows as the tiled kernel) and reads its MFMA fragments back from
-// LDS; the buffer is private to the wave, so no barrier is involved.  Weights still stream straight
-// into registers.  Requires K % (8 * 128) == 0.
+// A register-direct fragment load touches 16 different 128-byte lines (64 bytes of each) per
+// instruction, and the texture path handles such an instruction about four times slower than one that
+// covers 8 full lines; with more than a few activation rows that path, not HBM, becomes the limit.
+// Here every wave copies the weight rows AND the activation rows of its own K steps global -> LDS
+// with DMA loads of 8 full lines each (the same XOR-swizzled 128-byte rows as the tiled kernel) and
+// reads its MFMA fragments back from LDS.  The buffer is private to the wave, so no barrier is
+// involved: a batch is "issue all DMA, wait for this wave's loads, multiply".
 // ---------------------------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
@@ -190,9 +190,9 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 MSLK_AMD_DEVINL int row_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
 template <int MT, int NT, int U, int BIAS>
-__global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
+__global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
   constexpr int kWaves = 8;
-  constexpr int XBUF = U * MT * 2048;                       // bytes of staged activations per wave
+  constexpr int XBUF = U * (MT + NT) * 2048;                // bytes of staged operands per wave
   static_assert(XBUF >= NT * MT * 1024, "the reduction slot of a wave lives inside its staging buffer");
   __shared__ __attribute__((aligned(1024))) char lds[kWaves * XBUF];
   const int lane = threadIdx.x & 63;
@@ -202,12 +202,17 @@ __global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
   const int K = p.K;
   char* xbuf = lds + wave * XBUF;
 
-  const uint8_t* wp[NT];
+  // weight rows of this workgroup, as DMA source offsets (same lane -> (row, chunk) map as the activations)
+  uint32_t w_off[NT][2];
+  const uint8_t* w_base = p.wq + (int64_t)n0 * K;
 #pragma unroll
-  for (int tn = 0; tn < NT; ++tn) {
-    const int row = n0 + tn * 16 + i;
-    wp[tn] = p.wq + (int64_t)(row < p.N ? row : p.N - 1) * K + g * 16;
-  }
+  for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = 8 * h + (lane >> 3);
+      const int row = tn * 16 + r;
+      w_off[tn][h] = (uint32_t)(n0 + row < p.N ? row : p.N - 1 - n0) * (uint32_t)K + (((lane & 7) ^ row_swz(r)) << 4);
+    }
   // DMA source offsets: load h (0 / 1) of m-tile tm covers rows tm*16 + 8h + (lane >> 3); lane fetches the
   // logical 16-byte chunk that belongs at physical position (lane & 7) of its swizzled LDS row.
   uint32_t x_off[MT][2];
@@ -249,7 +254,6 @@ __global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
 
   const int KT = K / kStep;   // K % (8 * 128) == 0: every wave owns KT / 8 complete steps
   for (int kt0 = wave; kt0 < KT; kt0 += kWaves * U) {
-    v8i wf[U][NT];
     // Weights first: their HBM requests must not queue behind the (L2-resident) activation traffic.
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -257,11 +261,11 @@ __global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
       if (kt < KT) {           // wave-uniform
         const int k0 = kt * kStep;
 #pragma unroll
-        for (int tn = 0; tn < NT; ++tn) {
-          const v4i lo = load16_stream(wp[tn] + k0);
-          const v4i hi = load16_stream(wp[tn] + k0 + 64);
-          wf[u][tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
+        for (int tn = 0; tn < NT; ++tn)
+#pragma unroll
+          for (int h = 0; h < 2; ++h)
+            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(w_base + k0 + w_off[tn][h]),
+                                             (lds_ptr_t)(xbuf + ((u * (MT + NT) + MT + tn) * 2 + h) * 1024), 16, 0, 0);
       }
     }
 #pragma unroll
@@ -274,25 +278,34 @@ __global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
 #pragma unroll
           for (int h = 0; h < 2; ++h)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(p.xq + k0 + x_off[tm][h]),
-                                             (lds_ptr_t)(xbuf + ((u * MT + tm) * 2 + h) * 1024), 16, 0, 0);
+                                             (lds_ptr_t)(xbuf + ((u * (MT + NT) + tm) * 2 + h) * 1024), 16, 0, 0);
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMA has landed in its private buffer
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (kt0 + u * kWaves < KT) {
+        v8i wf[NT];
+#pragma unroll
+        for (int tn = 0; tn < NT; ++tn) {
+          const char* wt = xbuf + (u * (MT + NT) + MT + tn) * 2048;
+          const v4i lo = *reinterpret_cast<const v4i*>(wt + xr0);
+          const v4i hi = *reinterpret_cast<const v4i*>(wt + xr1);
+          wf[tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        }
 #pragma unroll
         for (int tm = 0; tm < MT; ++tm) {
-          const char* xt = xbuf + (u * MT + tm) * 2048;
+          const char* xt = xbuf + (u * (MT + NT) + tm) * 2048;
           const v4i lo = *reinterpret_cast<const v4i*>(xt + xr0);
           const v4i hi = *reinterpret_cast<const v4i*>(xt + xr1);
           const v8i xf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
           for (int tn = 0; tn < NT; ++tn)
-            acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[u][tn], xf, acc[tn][tm], 0, 0, 0, 0, 0, 0);
+            acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[tn], xf, acc[tn][tm], 0, 0, 0, 0, 0, 0);
         }
       }
     }
+    // the next batch re-uses the buffer: all LDS reads above have returned (their MFMAs were issued)
   }
 
   // Reduction across the 8 waves: each wave parks its partial tiles in its own (now dead) staging buffer.
@@ -321,12 +334,12 @@ __global__ __launch_bounds__(512) void skinny_xlds_kernel(GemmProblem p) {
 }
 
 template <int MT, int NT, int U>
-hipError_t launch_xlds(const GemmProblem& p, hipStream_t s) {
+hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
   const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
   switch (p.bias_dtype) {
-    case 0: skinny_xlds_kernel<MT, NT, U, 0><<<grid, 512, 0, s>>>(p); break;
-    case 1: skinny_xlds_kernel<MT, NT, U, 1><<<grid, 512, 0, s>>>(p); break;
-    default: skinny_xlds_kernel<MT, NT, U, 2><<<grid, 512, 0, s>>>(p); break;
+    case 0: skinny_lds_kernel<MT, NT, U, 0><<<grid, 512, 0, s>>>(p); break;
+    case 1: skinny_lds_kernel<MT, NT, U, 1><<<grid, 512, 0, s>>>(p); break;
+    default: skinny_lds_kernel<MT, NT, U, 2><<<grid, 512, 0, s>>>(p); break;
   }
   return hipGetLastError();
 }
@@ -340,10 +353,10 @@ bool skinny_supports(const GemmProblem& p) {
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
   if (!skinny_supports(p)) return hipErrorInvalidValue;
-  if (p.M > 4 && p.K % (8 * kStep) == 0) {   // activations through LDS
-    if (p.M <= 16) return launch_xlds<1, 1, 4>(p, s);
-    if (p.M <= 32) return launch_xlds<2, 1, 4>(p, s);
-    return launch_xlds<4, 2, 2>(p, s);
+  if (p.K % (8 * kStep) == 0) {   // both operands through LDS, all global traffic in full lines
+    if (p.M <= 16) return launch_lds<1, 1, 4>(p, s);
+    if (p.M <= 32) return launch_lds<2, 1, 1>(p, s);
+    return launch_lds<4, 2, 1>(p, s);
   }
   if (p.M <= 16) return launch_cfg<1, 1, 8>(p, s);
   if (p.M <= 32) return launch_cfg<2, 2, 4>(p, s);
