@@ -24,9 +24,9 @@ MSLK_AMD_DEVINL bool map_tile(int bid, int tiles_m, int tiles_n, int& tm, int& t
   return true;
 }
 
-template <int BM, int BN, int BIAS>
-__global__ __launch_bounds__(256) void dense_tiled_kernel(GemmProblem p, int tiles_m, int tiles_n) {
-  using TS = TileShape<BM, BN>;
+template <typename TS, int BIAS>
+__global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p, int tiles_m, int tiles_n) {
+  constexpr int BM = TS::kBM, BN = TS::kBN;
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
   int tm, tn;
   if (!map_tile(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
@@ -39,15 +39,16 @@ __global__ __launch_bounds__(256) void dense_tiled_kernel(GemmProblem p, int til
            p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K);
 }
 
-template <int BM, int BN>
+template <typename TS>
 hipError_t launch_tiled_shape(const GemmProblem& p, hipStream_t s) {
+  constexpr int BM = TS::kBM, BN = TS::kBN;
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const int grid = ((ntiles + kXcds - 1) / kXcds) * kXcds;
   switch (p.bias_dtype) {
-    case 0: dense_tiled_kernel<BM, BN, 0><<<grid, 256, 0, s>>>(p, tiles_m, tiles_n); break;
-    case 1: dense_tiled_kernel<BM, BN, 1><<<grid, 256, 0, s>>>(p, tiles_m, tiles_n); break;
-    default: dense_tiled_kernel<BM, BN, 2><<<grid, 256, 0, s>>>(p, tiles_m, tiles_n); break;
+    case 0: dense_tiled_kernel<TS, 0><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    case 1: dense_tiled_kernel<TS, 1><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    default: dense_tiled_kernel<TS, 2><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
   }
   return hipGetLastError();
 }
@@ -85,8 +86,8 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (!dense_tiled_supports(p)) return hipErrorInvalidValue;
   // 256 x 256 tiles once they give every CU work; 128 x 128 below that.
   const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-  if (big_tiles >= 192) return launch_tiled_shape<256, 256>(p, s);
-  return launch_tiled_shape<128, 128>(p, s);
+  if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>>(p, s);
+  return launch_tiled_shape<TileShape<128, 128>>(p, s);
 }
 
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s) {

@@ -1,6 +1,7 @@
 // LDS-tiled FP8 x FP8 -> fp32 MFMA main loop and fused rowwise-scale epilogue for gfx950.
 //
-// One workgroup of 256 lanes (4 wavefronts in a 2 x 2 grid) produces a BM x BN tile of
+// One workgroup (4 wavefronts in a 2 x 2 grid by default; 2 x 4 and 4 x 2 grids of 8 wavefronts compile
+// too but measured no faster) produces a BM x BN tile of
 //   Y[m, n] = bf16( (sum_k XQ[m, k] * WQ[n, k]) * x_scale[m] * w_scale[n] + bias[n] )
 // (reference math: csrc/gemm/ck/fp8_rowwise/kernels/fp8_rowwise_common.h:54-82,168-204; bias:
 //  csrc/gemm/cutlass/f8f8bf16_rowwise/f8f8bf16_rowwise_common.cuh:150-198).
@@ -28,17 +29,20 @@ namespace mslk_amd {
 
 constexpr int kBK = 128;  // bytes (= fp8 elements) of K per main-loop step
 
-template <int BM, int BN>
+template <int BM, int BN, int WAVES_M = 2, int WAVES_N = 2>
 struct TileShape {
   static constexpr int kBM = BM, kBN = BN;
-  static constexpr int FM = BM / 32;            // 16-row m fragments per wave (wave covers BM/2 rows)
-  static constexpr int FN = BN / 32;            // 16-row n fragments per wave
+  static constexpr int WM = WAVES_M, WN = WAVES_N;   // wave grid over the tile
+  static constexpr int NW = WAVES_M * WAVES_N;
+  static constexpr int NTHREADS = NW * 64;
+  static constexpr int FM = BM / WAVES_M / 16;  // 16-row m fragments per wave
+  static constexpr int FN = BN / WAVES_N / 16;  // 16-row n fragments per wave
   static constexpr int A_BYTES = BM * kBK;
   static constexpr int B_BYTES = BN * kBK;
   static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
   static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
-  static constexpr int LA = BM / 32;            // wave-level loads of the A tile per wave per step
-  static constexpr int LB = BN / 32;
+  static constexpr int LA = BM / 8 / NW;        // wave-level loads of the A tile per wave per step
+  static constexpr int LB = BN / 8 / NW;
 };
 
 MSLK_AMD_DEVINL int lds_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
@@ -144,10 +148,10 @@ struct GemmTile {
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
   MSLK_AMD_DEVINL static const char* a_tile_of(const char* stage) {
-    return stage + (wave_id() >> 1) * (TS::kBM / 2) * kBK;
+    return stage + (wave_id() / TS::WN) * (TS::kBM / TS::WM) * kBK;
   }
   MSLK_AMD_DEVINL static const char* b_tile_of(const char* stage) {
-    return stage + TS::A_BYTES + (wave_id() & 1) * (TS::kBN / 2) * kBK;
+    return stage + TS::A_BYTES + (wave_id() % TS::WN) * (TS::kBN / TS::WN) * kBK;
   }
   // First fragments of a K step: all XQ fragments and WQ fragment 0.
   MSLK_AMD_DEVINL void load_first_frags(const char* stage, v8i (&xf)[TS::FM], v8i& wf0) {
@@ -275,17 +279,17 @@ struct GemmTile {
   template <bool FULL>
   MSLK_AMD_DEVINL void epilogue_impl(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                      const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
-    constexpr int WN = TS::kBN / 2;              // columns per wave
+    constexpr int WN = TS::kBN / TS::WN;         // columns per wave
     constexpr int PITCH = WN * 2 + 16;           // bytes per staged row
     constexpr int BUF = 16 * PITCH;
     constexpr int CH = WN / 8;                   // 16-byte chunks per row (16 for BN = 256)
     constexpr int RPI = 64 / CH;                 // rows written per store instruction
     const int lane = threadIdx.x & 63, wave = wave_id();
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave / TS::WN, wn = wave % TS::WN;
     const int j = lane & 15, q = lane >> 4;
     char* buf = lds + wave * 2 * BUF;
     const int n_base = wn * WN;
-    const int m_base = wm * (TS::kBM / 2);
+    const int m_base = wm * (TS::kBM / TS::WM);
     const bool vec_store = (N & 7) == 0;
 
     float wsv[TS::FN][4], bv[TS::FN][4];
