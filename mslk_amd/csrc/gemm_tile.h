@@ -354,6 +354,14 @@ struct GemmTile {
           if (mm >= m_rem || nn >= n_rem) continue;
           if (vec_store && nn + 7 < n_rem) {
             store16_stream(dst, val);
+          } else if ((N & 1) == 0) {   // rows are 4-byte aligned: store bf16 pairs
+            const uint32_t w[4] = {val.x, val.y, val.z, val.w};
+            uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if (nn + 2 * e + 1 < n_rem) d32[e] = w[e];
+              else if (nn + 2 * e < n_rem) dst[2 * e] = (uint16_t)w[e];
+            }
           } else {
             const uint32_t w[4] = {val.x, val.y, val.z, val.w};
 #pragma unroll

@@ -43,7 +43,7 @@ SHAPES = [
     (300, 520, 640), (257, 255, 384), (129, 1000, 4096), (512, 768, 144), (512, 512, 16), (384, 130, 2064),
     (100, 100, 100), (65, 33, 17), (70, 64, 1), (1, 8192, 8192), (4, 8192, 8192), (16, 8192, 8192), (64, 8192, 8192),
     (3, 1000, 272), (17, 260, 4096), (33, 48, 512), (48, 16, 128), (64, 15, 256), (1, 1, 16), (2, 7, 24),
-    (8, 100, 1024), (33, 48, 2048), (50, 1000, 3072), (64, 15, 1024), (5, 8200, 5120), (20, 513, 9216),
+    (300, 517, 256), (513, 1030, 384), (8, 100, 1024), (33, 48, 2048), (50, 1000, 3072), (64, 15, 1024), (5, 8200, 5120), (20, 513, 9216),
 ]
 
 
