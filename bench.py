@@ -333,7 +333,34 @@ def main():
         f4 = 2.0 * 8192 * 8192 * 5120
         extras["grouped_cfg4_16x8192x5120"] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12,
                                                 "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS, "counts": wl4.counts}
-        del wq4, wl4
+        # the same experts through the device-resident group layouts (no host knowledge of the sizes),
+        # and as a uniform batch of 16 x [512 x 8192 x 5120] (same FLOPs, no ragged tiles)
+        WQ4, WS4 = torch.stack(wq4), torch.stack(ws4)
+        del wq4, ws4, call4
+        y4 = torch.empty(8192, 8192, dtype=torch.bfloat16, device=dev)
+        sizes = torch.tensor(wl4.counts, dtype=torch.int64, device=dev)
+        ends = sizes.cumsum(0).to(torch.int32)
+        L = api.L
+
+        def stacked_call():
+            api.check(L.mslk_amd_f8f8bf16_rowwise_grouped_stacked(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
+                                                                  sizes.data_ptr(), 16, 8192, 8192, 5120, y4.data_ptr(), api.stream))
+
+        def offsets_call():
+            api.check(L.mslk_amd_f8f8bf16_rowwise_grouped_mm(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
+                                                             ends.data_ptr(), 1, 16, 8192, 8192, 5120, y4.data_ptr(), api.stream))
+
+        def batched_call():
+            api.check(L.mslk_amd_f8f8bf16_rowwise_batched(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
+                                                          None, 0, 16, 512, 8192, 5120, y4.data_ptr(), api.stream))
+
+        for name, call in (("grouped_stacked_cfg4", stacked_call), ("grouped_mm_2d3d_cfg4", offsets_call),
+                           ("batched_16x512x8192x5120", batched_call)):
+            for _ in range(3):
+                call()
+            ms = _median_events_ms(lambda i: call(), 10)
+            extras[name] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12, "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS}
+        del WQ4, wl4
 
     # ---------------------------------------------------------------- CPU baseline
     cpu = None

@@ -92,6 +92,43 @@ int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, co
                                               int64_t total_M, int64_t N, int64_t K, void* y, void* stream);
 
 /*
+ * Grouped GEMM in the torch._grouped_mm calling convention: group boundaries are int32 cumulative
+ * END offsets in DEVICE memory (no host sync; graph-safe).  Replaces
+ * mslk::gemm::f8f8bf16_rowwise_grouped_mm (reference: csrc/gemm/gemm_ops.cpp:35-36,
+ * csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:720-845; the per-group pointer
+ * arithmetic restates set_kernel_args, same file 161-296).  `layout` selects the varying dimension;
+ * M, N, K are the full tensor extents (the varying one is the total over groups):
+ *   MSLK_AMD_GROUPS_M_OFFSETS  "2D-3D": xq [M, K], wq [G, N, K], x_scale [M], w_scale [G, N], y [M, N];
+ *                              group g owns rows offsets[g-1] .. offsets[g] of xq / y.
+ *   MSLK_AMD_GROUPS_N_OFFSETS  "3D-2D": xq [G, M, K], wq [N, K], x_scale [G, M], w_scale [N], y [M, N];
+ *                              group g owns rows offsets[g-1] .. offsets[g] of wq = those columns of y.
+ *   MSLK_AMD_GROUPS_K_OFFSETS  "2D-2D": xq [M, K], wq [N, K], x_scale [G*M], w_scale [G*N], y [G, M, N];
+ *                              group g multiplies the K slice offsets[g-1] .. offsets[g] of both.
+ *   MSLK_AMD_GROUPS_UNIFORM    "3D-3D": xq [G, M, K], wq [G, N, K], x_scale [G, M], w_scale [G, N],
+ *                              y [G, M, N]; offsets must be NULL.
+ * Rows / columns beyond offsets[G-1] are left untouched; an empty K slice writes zeros.  Offsets that
+ * decrease or exceed the tensor extent make the affected workgroups write nothing.
+ */
+#define MSLK_AMD_GROUPS_M_OFFSETS 1
+#define MSLK_AMD_GROUPS_N_OFFSETS 2
+#define MSLK_AMD_GROUPS_K_OFFSETS 3
+#define MSLK_AMD_GROUPS_UNIFORM 4
+int mslk_amd_f8f8bf16_rowwise_grouped_mm(const void* xq, const void* wq, const float* x_scale,
+                                         const float* w_scale, const int32_t* offsets_dev, int layout, int G,
+                                         int64_t M, int64_t N, int64_t K, void* y, void* stream);
+
+/*
+ * Batched rowwise FP8 GEMM: Y[b] = bf16(XQ[b] . WQ[b]^T * x_scale[b][:,None] * w_scale[b][None,:] + bias[b]).
+ * Replaces mslk::gemm::f8f8bf16_rowwise_batched (reference: csrc/gemm/gemm_ops.cpp:95-96,
+ * csrc/gemm/ck/fp8_rowwise_batched/fp8_rowwise_batched_gemm.hip:199-254).
+ *   xq [B, M, K], wq [B, N, K], x_scale [B, M], w_scale [B, N], bias NULL or [B, N] (layout of
+ *   csrc/gemm/cutlass/f8f8bf16_rowwise_batched/f8f8bf16_rowwise_batched_common.cuh:272-275), y [B, M, N].
+ */
+int mslk_amd_f8f8bf16_rowwise_batched(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                                      const void* bias, int bias_dtype, int64_t B, int64_t M, int64_t N,
+                                      int64_t K, void* y, void* stream);
+
+/*
  * Self-test helper: converts n fp32 values to e4m3fn with the same device routine the quantizer
  * uses (hardware v_cvt_pk_fp8_f32 plus the NaN fix-up for |v| > 464).  Used by the parity tests to
  * sweep the conversion against the oracle; no counterpart in the reference.

@@ -28,6 +28,10 @@ SIGNATURES = {
                                                   POINTER(c_int64), POINTER(c_int64), c_void_p]),
     "mslk_amd_f8f8bf16_rowwise_grouped_stacked": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                                           c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "mslk_amd_f8f8bf16_rowwise_grouped_mm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                                     c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "mslk_amd_f8f8bf16_rowwise_batched": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
+                                                  c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "mslk_amd_debug_cast_e4m3fn": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),
 }
 

@@ -124,12 +124,49 @@ int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, co
   if (!y) return fail("f8f8bf16_rowwise_grouped_stacked: null output");
   if (K == 0) return check_hip(launch_fill_zero_bf16((uint16_t*)y, total_M * N, s), "zero fill");
   if (!xq || !wq || !x_scale || !w_scale || !m_sizes_dev) return fail("f8f8bf16_rowwise_grouped_stacked: null pointer");
-  if (!grouped_tiled_supports((int)N, (int)K) || reinterpret_cast<uintptr_t>(xq) % 16 || reinterpret_cast<uintptr_t>(wq) % 16 ||
-      reinterpret_cast<uintptr_t>(y) % 16)
-    return fail("f8f8bf16_rowwise_grouped_stacked: K must be a multiple of 16 and XQ/WQ 16-byte aligned (K=%lld)", (long long)K);
-  return check_hip(launch_grouped_stacked((const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, m_sizes_dev, G,
-                                          total_M, (int)N, (int)K, (uint16_t*)y, s),
-                   "grouped stacked launch");
+  DeviceGroups p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, nullptr, (uint16_t*)y, m_sizes_dev, G,
+                 (int)total_M, (int)N, (int)K, 0, 0};
+  return check_hip(launch_device_groups(p, kGroupsSizesM, s), "grouped stacked launch");
+}
+
+int mslk_amd_f8f8bf16_rowwise_grouped_mm(const void* xq, const void* wq, const float* x_scale,
+                                         const float* w_scale, const int32_t* offsets_dev, int layout, int G,
+                                         int64_t M, int64_t N, int64_t K, void* y, void* stream) {
+  if (layout < MSLK_AMD_GROUPS_M_OFFSETS || layout > MSLK_AMD_GROUPS_UNIFORM)
+    return fail("f8f8bf16_rowwise_grouped_mm: unknown group layout code %d", layout);
+  if (G < 0 || M < 0 || N < 0 || K < 0) return fail("f8f8bf16_rowwise_grouped_mm: negative dimension");
+  if (M > kIntMax || N > kIntMax || K > kIntMax) return fail("f8f8bf16_rowwise_grouped_mm: dimension exceeds 2^31-1");
+  const bool uniform = layout == MSLK_AMD_GROUPS_UNIFORM;
+  if (uniform != (offsets_dev == nullptr))
+    return fail(uniform ? "f8f8bf16_rowwise_grouped_mm: offsets must be NULL for the uniform layout"
+                        : "f8f8bf16_rowwise_grouped_mm: offsets are required for this layout");
+  hipStream_t s = (hipStream_t)stream;
+  if (G == 0 || M == 0 || N == 0) return 0;
+  if (!y) return fail("f8f8bf16_rowwise_grouped_mm: null output");
+  const bool stacked_out = layout == MSLK_AMD_GROUPS_K_OFFSETS || uniform;   // y is [G, M, N]
+  if (stacked_out && (double)G * (double)M * (double)N > 9.0e18) return fail("f8f8bf16_rowwise_grouped_mm: output too large");
+  // K == 0 needs no special case: every tile a group owns is written with the empty sum.
+  if ((K > 0 && (!xq || !wq)) || !x_scale || !w_scale) return fail("f8f8bf16_rowwise_grouped_mm: null pointer");
+  DeviceGroups p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, nullptr, (uint16_t*)y, offsets_dev, G,
+                 (int)M, (int)N, (int)K, 0, 0};
+  return check_hip(launch_device_groups(p, layout, s), "grouped_mm launch");
+}
+
+int mslk_amd_f8f8bf16_rowwise_batched(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                                      const void* bias, int bias_dtype, int64_t B, int64_t M, int64_t N,
+                                      int64_t K, void* y, void* stream) {
+  if (B < 0 || M < 0 || N < 0 || K < 0) return fail("f8f8bf16_rowwise_batched: negative dimension");
+  if (B > kIntMax || M > kIntMax || N > kIntMax || K > kIntMax) return fail("f8f8bf16_rowwise_batched: dimension exceeds 2^31-1");
+  if (bias_dtype < 0 || bias_dtype > 2) return fail("f8f8bf16_rowwise_batched: bad bias dtype code %d", bias_dtype);
+  if ((bias_dtype != 0) != (bias != nullptr)) return fail("f8f8bf16_rowwise_batched: bias pointer and bias dtype disagree");
+  hipStream_t s = (hipStream_t)stream;
+  if (B == 0 || M == 0 || N == 0) return 0;
+  if (!y) return fail("f8f8bf16_rowwise_batched: null output");
+  if ((double)B * (double)M * (double)N > 9.0e18) return fail("f8f8bf16_rowwise_batched: output too large");
+  if ((K > 0 && (!xq || !wq)) || !x_scale || !w_scale) return fail("f8f8bf16_rowwise_batched: null pointer");
+  DeviceGroups p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y, nullptr, (int)B,
+                 (int)M, (int)N, (int)K, bias_dtype, 0};
+  return check_hip(launch_device_groups(p, kGroupsUniform, s), "batched launch");
 }
 
 int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stream) {

@@ -4,9 +4,12 @@
 //   * TensorList API (reference csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:481-559):
 //     shapes are host-known, so the group descriptors and their tile prefix sums travel in the
 //     kernel-argument block (no device-side setup launches, no workspace, graph-safe).
-//   * Stacked API (same file, 607-655): group sizes live in device memory; every workgroup walks the
-//     G sizes (L2-resident) to find its tile, and the grid is sized for the worst case
-//     ceil(total_M / BM) + G row tiles, so no host synchronisation is needed.
+//   * Stacked API (same file, 607-655) and the offsets API (f8f8bf16_rowwise_grouped_mm, same file
+//     720-845; its device-side layouts are restated from set_kernel_args, 161-296): group extents live
+//     in device memory; every workgroup walks the G entries (L2-resident) to find its tile, and the
+//     grid is sized for the worst case (one partial tile per group), so no host synchronisation is
+//     needed.  The batched op (csrc/gemm/ck/fp8_rowwise_batched/fp8_rowwise_batched_gemm.hip:199-254)
+//     is the uniform layout.
 // Empty groups own no tiles and are never touched.
 #include "gemm_tile.h"
 #include "kernels.h"
@@ -46,37 +49,173 @@ __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
            d.y + (int64_t)m0 * d.N + n0, d.M - m0, d.N - n0, d.N, d.K);
 }
 
-template <int BM, int BN>
-__global__ __launch_bounds__(256) void grouped_stacked_kernel(const uint8_t* xq, const uint8_t* wq, const float* xs,
-                                                              const float* ws, const int64_t* m_sizes, int G,
-                                                              int64_t total_M, int N, int K, uint16_t* y) {
+// Groups whose extents live in device memory (or are uniform).  `layout` says which dimension varies
+// per group and how it is encoded; the fixed dimensions come from p.M / p.N / p.K, where the varying
+// one holds the total over all groups.
+//   kGroupsSizesM    int64 sizes of the row blocks of XQ [sum M, K]; WQ [G, N, K]; Y [sum M, N]
+//   kGroupsOffsetsM  int32 cumulative ends of the same row blocks
+//   kGroupsOffsetsN  XQ [G, M, K]; int32 cumulative ends of row blocks of WQ [sum N, K]; Y [M, sum N]
+//   kGroupsOffsetsK  XQ [M, sum K], WQ [N, sum K]; int32 cumulative ends of K slices; Y [G, M, N]
+//   kGroupsUniform   XQ [G, M, K], WQ [G, N, K], Y [G, M, N]
+// Scales follow the operand they belong to ([sum M] or [G, M]; [sum N] or [G, N]).
+struct GroupSpan {
+  int gi;        // group
+  int64_t o0;    // first index of the group along the varying dimension
+  int len;       // extent of the group along the varying dimension
+  int t;         // tile index inside the group
+};
+
+template <int LAYOUT, int BM, int BN>
+MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  if constexpr (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK) {
+    const int per = tiles_m * tiles_n;
+    sp.gi = t / per;
+    sp.t = t - sp.gi * per;
+    if (sp.gi >= p.G) return false;
+    if constexpr (LAYOUT == kGroupsUniform) {
+      sp.o0 = 0;
+      sp.len = 0;
+      return true;
+    } else {
+      const int32_t* off = static_cast<const int32_t*>(p.layout);
+      const int64_t b = sp.gi ? off[sp.gi - 1] : 0, e = off[sp.gi];
+      sp.o0 = b;
+      sp.len = (int)(e - b);
+      return b >= 0 && e >= b && e <= p.K;
+    }
+  } else {
+    const int fixed_tiles = LAYOUT == kGroupsOffsetsN ? tiles_m : tiles_n;
+    const int blk = LAYOUT == kGroupsOffsetsN ? BN : BM;
+    const int64_t total = LAYOUT == kGroupsOffsetsN ? p.N : p.M;
+    int64_t b = 0;
+    for (int gi = 0; gi < p.G; ++gi) {
+      int64_t len;
+      if constexpr (LAYOUT == kGroupsSizesM) {
+        len = static_cast<const int64_t*>(p.layout)[gi];
+      } else {
+        len = (int64_t) static_cast<const int32_t*>(p.layout)[gi] - b;
+      }
+      if (len < 0 || b + len > total) return false;   // inconsistent group data: touch nothing
+      const int64_t tiles = ((len + blk - 1) / blk) * fixed_tiles;
+      if (t < tiles) {
+        sp.gi = gi; sp.o0 = b; sp.len = (int)len; sp.t = t;
+        return true;
+      }
+      t -= (int)tiles;
+      b += len;
+    }
+    return false;
+  }
+}
+
+// Scalar tile for operands the DMA path cannot fetch (row starts or K extents that are not multiples
+// of 16 bytes): one lane per output element, sequential K.
+template <int BM, int BN, int BIAS>
+MSLK_AMD_DEVINL void slow_tile(const uint8_t* a, const uint8_t* b, const float* xs, const float* ws,
+                               const void* bias, uint16_t* y, int m_rem, int n_rem, int ldc, int K, int64_t ld) {
+  const int mt = m_rem < BM ? m_rem : BM, nt = n_rem < BN ? n_rem : BN;
+  for (int idx = threadIdx.x; idx < mt * nt; idx += 256) {
+    const int m = idx / nt, n = idx - m * nt;
+    const uint8_t* ar = a + m * ld;
+    const uint8_t* br = b + n * ld;
+    float acc = 0.f;
+    for (int k = 0; k < K; ++k)
+      acc += __builtin_amdgcn_cvt_f32_fp8((int)ar[k], 0) * __builtin_amdgcn_cvt_f32_fp8((int)br[k], 0);
+    float v = (acc * xs[m]) * ws[n];
+    if constexpr (BIAS == 1) v += static_cast<const float*>(bias)[n];
+    if constexpr (BIAS == 2) v += bf16_bits_to_f32(static_cast<const uint16_t*>(bias)[n]);
+    y[(int64_t)m * ldc + n] = (uint16_t)f32_to_bf16_bits(v);
+  }
+}
+
+template <int LAYOUT, int BM, int BN, int BIAS>
+__global__ __launch_bounds__(256) void grouped_device_kernel(DeviceGroups p) {
   using TS = TileShape<BM, BN>;
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
-  const int tiles_n = (N + BN - 1) / BN;
   int t = blockIdx.x;
-  int64_t row0 = 0;
-  int gi = 0, Mg = 0;
-  for (; gi < G; ++gi) {
-    const int64_t mg = m_sizes[gi];
-    const int tiles = (int)((mg + BM - 1) / BM) * tiles_n;
-    if (t < tiles) { Mg = (int)mg; break; }
-    t -= tiles;
-    row0 += mg;
+  if constexpr (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK) {
+    // The tile count is known on the host: XCD x works on a contiguous slice of the tile list.
+    const int total = p.G * ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+    const int per_xcd = (total + kXcds - 1) / kXcds;
+    t = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
+    if (t >= total) return;
   }
-  if (gi >= G || row0 + Mg > total_M) return;
+  GroupSpan sp;
+  if (!find_group<LAYOUT, BM, BN>(p, t, sp)) return;
+  const int64_t g = sp.gi, M = p.M, N = p.N, K = p.K;
+  const int Mg = (LAYOUT == kGroupsSizesM || LAYOUT == kGroupsOffsetsM) ? sp.len : p.M;
+  const int Ng = LAYOUT == kGroupsOffsetsN ? sp.len : p.N;
+  const int Kg = LAYOUT == kGroupsOffsetsK ? sp.len : p.K;
   int tm, tn;
-  local_tile(t, (Mg + BM - 1) / BM, tiles_n, tm, tn);
-  const int m0 = tm * BM, n0 = tn * BN;
-  GemmTile<TS, 0> tile;
-  tile.run(lds, xq + (row0 + m0) * K, wq + ((int64_t)gi * N + n0) * K, xs + row0 + m0, ws + (int64_t)gi * N + n0,
-           nullptr, y + (row0 + m0) * N + n0, Mg - m0, N - n0, N, K);
+  local_tile(sp.t, (Mg + BM - 1) / BM, (Ng + BN - 1) / BN, tm, tn);
+  const int64_t m0 = tm * BM, n0 = tn * BN;
+  const uint8_t *a, *b;
+  const float *xs, *ws;
+  uint16_t* y;
+  if constexpr (LAYOUT == kGroupsSizesM || LAYOUT == kGroupsOffsetsM) {
+    a = p.xq + (sp.o0 + m0) * K;      b = p.wq + (g * N + n0) * K;
+    xs = p.xs + sp.o0 + m0;           ws = p.ws + g * N + n0;
+    y = p.y + (sp.o0 + m0) * N + n0;
+  } else if constexpr (LAYOUT == kGroupsOffsetsN) {
+    a = p.xq + (g * M + m0) * K;      b = p.wq + (sp.o0 + n0) * K;
+    xs = p.xs + g * M + m0;           ws = p.ws + sp.o0 + n0;
+    y = p.y + m0 * N + sp.o0 + n0;
+  } else if constexpr (LAYOUT == kGroupsOffsetsK) {
+    a = p.xq + m0 * K + sp.o0;        b = p.wq + n0 * K + sp.o0;
+    xs = p.xs + g * M + m0;           ws = p.ws + g * N + n0;
+    y = p.y + (g * M + m0) * N + n0;
+  } else {
+    a = p.xq + (g * M + m0) * K;      b = p.wq + (g * N + n0) * K;
+    xs = p.xs + g * M + m0;           ws = p.ws + g * N + n0;
+    y = p.y + (g * M + m0) * N + n0;
+  }
+  const int m_rem = Mg - (int)m0, n_rem = Ng - (int)n0;
+  const void* bias = nullptr;
+  if constexpr (BIAS == 1) bias = static_cast<const float*>(p.bias) + g * N + n0;
+  if constexpr (BIAS == 2) bias = static_cast<const uint16_t*>(p.bias) + g * N + n0;
+  bool slow = p.unaligned != 0;
+  if constexpr (LAYOUT == kGroupsOffsetsK) slow = slow || (sp.o0 & 15) != 0 || (Kg & 15) != 0;
+  if (slow) {   // Kg == 0 needs no special case on either path: the sum is empty
+    slow_tile<BM, BN, BIAS>(a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, K);
+    return;
+  }
+  GemmTile<TS, BIAS> tile;
+  tile.run(lds, a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, (uint32_t)p.K);
+}
+
+template <int LAYOUT, int BM, int BN, int BIAS>
+hipError_t launch_device_shape(const DeviceGroups& p, hipStream_t s) {
+  const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  int64_t grid;
+  if (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK) {
+    grid = (p.G * tiles_m * tiles_n + kXcds - 1) / kXcds * kXcds;
+  } else if (LAYOUT == kGroupsOffsetsN) {
+    grid = tiles_m * (tiles_n + p.G);   // every group may end in a partial tile
+  } else {
+    grid = (tiles_m + p.G) * tiles_n;
+  }
+  if (grid <= 0) return hipSuccess;
+  if (grid > 2147483647) return hipErrorInvalidValue;
+  grouped_device_kernel<LAYOUT, BM, BN, BIAS><<<(unsigned)grid, 256, 0, s>>>(p);
+  return hipGetLastError();
+}
+
+template <int LAYOUT, int BIAS>
+hipError_t launch_device_layout(const DeviceGroups& p, hipStream_t s) {
+  // Tile shape from the average group: 256 x 256 once such tiles give every CU work.
+  const int64_t G = p.G > 0 ? p.G : 1;
+  int64_t Mg = p.M, Ng = p.N;
+  if (LAYOUT == kGroupsSizesM || LAYOUT == kGroupsOffsetsM) Mg = (p.M + G - 1) / G;
+  if (LAYOUT == kGroupsOffsetsN) Ng = (p.N + G - 1) / G;
+  const int64_t big = G * ((Mg + 255) / 256) * ((Ng + 255) / 256);
+  const int64_t pad = ((Mg + 255) / 256 * 256) * ((Ng + 255) / 256 * 256);
+  const bool use_big = big >= 192 && pad * 4 <= Mg * Ng * 5;   // at most 25 % padding
+  if (use_big) return launch_device_shape<LAYOUT, 256, 256, BIAS>(p, s);
+  return launch_device_shape<LAYOUT, 128, 128, BIAS>(p, s);
 }
 
 }  // namespace
-
-bool grouped_tiled_supports(int N, int K) {
-  return K % 16 == 0 && K >= 16 && (int64_t)256 * K < (int64_t(1) << 32) && N >= 1;
-}
 
 hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s) {
   if (t.total_tiles <= 0) return hipSuccess;
@@ -85,14 +224,26 @@ hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s) {
   return hipGetLastError();
 }
 
-hipError_t launch_grouped_stacked(const uint8_t* xq, const uint8_t* wq, const float* xs, const float* ws,
-                                  const int64_t* m_sizes, int G, int64_t total_M, int N, int K, uint16_t* y,
-                                  hipStream_t s) {
-  constexpr int BM = 256, BN = 256;
-  const int64_t tiles = ((total_M + BM - 1) / BM + G) * ((N + BN - 1) / BN);
-  if (tiles <= 0) return hipSuccess;
-  grouped_stacked_kernel<BM, BN><<<(unsigned)tiles, 256, 0, s>>>(xq, wq, xs, ws, m_sizes, G, total_M, N, K, y);
-  return hipGetLastError();
+// Whether every operand row of the problem can be fetched by the 16-byte DMA path.
+static bool device_groups_aligned(const DeviceGroups& p) {
+  return p.K % 16 == 0 && (int64_t)256 * p.K < (int64_t(1) << 32) &&
+         reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0;
+}
+
+hipError_t launch_device_groups(const DeviceGroups& in, int layout, hipStream_t s) {
+  DeviceGroups p = in;
+  p.unaligned = device_groups_aligned(p) ? 0 : 1;
+  switch (layout) {
+    case kGroupsSizesM: return launch_device_layout<kGroupsSizesM, 0>(p, s);
+    case kGroupsOffsetsM: return launch_device_layout<kGroupsOffsetsM, 0>(p, s);
+    case kGroupsOffsetsN: return launch_device_layout<kGroupsOffsetsN, 0>(p, s);
+    case kGroupsOffsetsK: return launch_device_layout<kGroupsOffsetsK, 0>(p, s);
+    case kGroupsUniform:
+      if (p.bias_dtype == 1) return launch_device_layout<kGroupsUniform, 1>(p, s);
+      if (p.bias_dtype == 2) return launch_device_layout<kGroupsUniform, 2>(p, s);
+      return launch_device_layout<kGroupsUniform, 0>(p, s);
+  }
+  return hipErrorInvalidValue;
 }
 
 }  // namespace mslk_amd

@@ -72,7 +72,8 @@ struct GemmTile {
   const uint8_t* b_base;    // WQ + n0 * K
 
   // xq/wq point at row m0 / n0 of the operands; rows_a / rows_b = valid rows from there (>= 1).
-  MSLK_AMD_DEVINL void init(const uint8_t* xq_tile, const uint8_t* wq_tile, int rows_a, int rows_b, int K) {
+  // `ld` = bytes between consecutive rows of XQ and of WQ (equal to K unless the operands are K slices).
+  MSLK_AMD_DEVINL void init(const uint8_t* xq_tile, const uint8_t* wq_tile, int rows_a, int rows_b, uint32_t ld) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     a_base = xq_tile;
     b_base = wq_tile;
@@ -81,14 +82,14 @@ struct GemmTile {
       const int row = (wave * TS::LA + i) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swz(row);
       const int rc = row < rows_a ? row : rows_a - 1;   // clamp: edge tiles re-read the last row
-      a_off[i] = (uint32_t)rc * (uint32_t)K + chunk * 16;
+      a_off[i] = (uint32_t)rc * ld + chunk * 16;
     }
 #pragma unroll
     for (int i = 0; i < TS::LB; ++i) {
       const int row = (wave * TS::LB + i) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swz(row);
       const int rc = row < rows_b ? row : rows_b - 1;
-      b_off[i] = (uint32_t)rc * (uint32_t)K + chunk * 16;
+      b_off[i] = (uint32_t)rc * ld + chunk * 16;
     }
   }
 
@@ -224,9 +225,16 @@ struct GemmTile {
 
   // Whole tile: K loop + epilogue.  m_rem / n_rem = valid rows / columns of this tile (>= 1).
   // xq_tile / wq_tile / xs / ws / bias / y are already offset to the tile's first row and column.
+  // N = elements between consecutive rows of Y; K = bytes of each operand row to consume;
+  // ld = bytes between consecutive operand rows.
   MSLK_AMD_DEVINL void run(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, const float* xs,
                            const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K) {
-    init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, K);
+    run(lds, xq_tile, wq_tile, xs, ws, bias, y, m_rem, n_rem, N, K, (uint32_t)K);
+  }
+  MSLK_AMD_DEVINL void run(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, const float* xs,
+                           const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K,
+                           uint32_t ld) {
+    init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
     v4f acc[TS::FN][TS::FM];
 #pragma unroll
     for (int tn = 0; tn < TS::FN; ++tn)
@@ -270,7 +278,11 @@ struct GemmTile {
                                 const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     // Tiles whose columns are all valid (the common case, also for the ragged last row tile of an MoE
     // group) take a path whose only bounds logic is one row test per store instruction.
-    const bool full = n_rem >= TS::kBN && (N & 7) == 0;
+    // 16-byte accesses need 16-byte aligned rows of Y and aligned scale / bias vectors (a tile that
+    // starts at a column offset inside a wider output may have neither).
+    const bool vec16 = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const bool full = n_rem >= TS::kBN && vec16 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
+                      (BIAS == 0 || (reinterpret_cast<uintptr_t>(bias) & (BIAS == 1 ? 15 : 7)) == 0);
     if (full) epilogue_impl<true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
     else epilogue_impl<false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
   }
@@ -290,7 +302,8 @@ struct GemmTile {
     char* buf = lds + wave * 2 * BUF;
     const int n_base = wn * WN;
     const int m_base = wm * (TS::kBM / TS::WM);
-    const bool vec_store = (N & 7) == 0;
+    const bool vec_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    const bool pair_store = (N & 1) == 0 && (reinterpret_cast<uintptr_t>(y) & 3) == 0;
 
     float wsv[TS::FN][4], bv[TS::FN][4];
 #pragma unroll
@@ -354,7 +367,7 @@ struct GemmTile {
           if (mm >= m_rem || nn >= n_rem) continue;
           if (vec_store && nn + 7 < n_rem) {
             store16_stream(dst, val);
-          } else if ((N & 1) == 0) {   // rows are 4-byte aligned: store bf16 pairs
+          } else if (pair_store) {   // rows are 4-byte aligned: store bf16 pairs
             const uint32_t w[4] = {val.x, val.y, val.z, val.w};
             uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);
 #pragma unroll

@@ -46,10 +46,29 @@ struct GroupTable {
   int count;
   int total_tiles;
 };
-bool grouped_tiled_supports(int N, int K);
 hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s);
-hipError_t launch_grouped_stacked(const uint8_t* xq, const uint8_t* wq, const float* xs, const float* ws,
-                                  const int64_t* m_sizes, int G, int64_t total_M, int N, int K, uint16_t* y,
-                                  hipStream_t s);
+
+// Groups described in device memory (or uniform); see gemm_grouped.hip for the layouts.
+enum GroupLayout : int {
+  kGroupsSizesM = 0,
+  kGroupsOffsetsM = 1,
+  kGroupsOffsetsN = 2,
+  kGroupsOffsetsK = 3,
+  kGroupsUniform = 4,
+};
+struct DeviceGroups {
+  const uint8_t* xq;
+  const uint8_t* wq;
+  const float* xs;
+  const float* ws;
+  const void* bias;     // [G, N], uniform layout only
+  uint16_t* y;
+  const void* layout;   // int64 sizes, int32 cumulative ends, or nullptr
+  int G;
+  int M, N, K;          // the varying dimension holds the total over all groups
+  int bias_dtype;       // 0 none, 1 fp32, 2 bf16
+  int unaligned;        // set by the launcher: operands need the scalar tile path
+};
+hipError_t launch_device_groups(const DeviceGroups& p, int layout, hipStream_t s);
 
 }  // namespace mslk_amd

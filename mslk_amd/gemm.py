@@ -1,6 +1,6 @@
 """`torch.ops.mslk.*` rowwise FP8 GEMM operators backed by the gfx950 HIP kernels.
 
-The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-34,37-42), so callers written
+The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-42,95-96), so callers written
 against `torch.ops.mslk.f8f8bf16_rowwise` etc. run unchanged.  When the reference's own library has
 already defined a schema, only the GPU ("CUDA" dispatch key) kernel is replaced -- the same seam
 the reference's Python kernels use (mslk/gemm/flydsl/preshuffle_gemm.py:433-475).
@@ -29,6 +29,8 @@ _SCHEMAS = {
     "f8f8bf16_rowwise_grouped": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor[]",
     "f8f8bf16_rowwise_grouped_cat": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor",
     "f8f8bf16_rowwise_grouped_stacked": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor M_sizes) -> Tensor",
+    "f8f8bf16_rowwise_grouped_mm": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? offsets, Tensor(a!) output) -> Tensor",
+    "f8f8bf16_rowwise_batched": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True, Tensor(a!)? output=None) -> Tensor",
 }
 
 _library = torch.library.Library("mslk", "FRAGMENT")
@@ -211,6 +213,121 @@ def f8f8bf16_rowwise_grouped_stacked(XQ, WQ, x_scale, w_scale, M_sizes) -> torch
     return Y
 
 
+# group layout codes of mslk_amd_f8f8bf16_rowwise_grouped_mm (include/mslk_amd.h)
+_GROUPS_M_OFFSETS, _GROUPS_N_OFFSETS, _GROUPS_K_OFFSETS, _GROUPS_UNIFORM = 1, 2, 3, 4
+
+
+def f8f8bf16_rowwise_grouped_mm(XQ, WQ, x_scale, w_scale, offsets, output) -> torch.Tensor:
+    """Grouped GEMM in the torch._grouped_mm convention (fp8_rowwise_grouped_gemm.hip:720-845): the
+    ranks of XQ / WQ select which dimension varies per group, `offsets` (int32, on the GPU, never
+    read on the host) holds the cumulative group ends along it, and the result is written into
+    `output`, which is returned.
+
+      XQ [total_M, K], WQ [G, N, K]   offsets over M   output [total_M, N]
+      XQ [G, M, K],    WQ [total_N, K] offsets over N   output [M, total_N]
+      XQ [G, M, K],    WQ [G, N, K]    no offsets       output [G, M, N]
+      XQ [M, total_K], WQ [N, total_K] offsets over K   output [G, M, N]
+    """
+    _check(XQ.is_cuda and XQ.is_contiguous() and WQ.is_cuda and WQ.is_contiguous(), "XQ/WQ must be contiguous GPU tensors")
+    _check(XQ.dtype == WQ.dtype, f"XQ and WQ dtypes must match, got {XQ.dtype} vs {WQ.dtype}")
+    _check(XQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ.dtype}")
+    _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
+    _check(x_scale.is_contiguous() and w_scale.is_contiguous(), "scales must be contiguous")
+
+    def need_offsets(what):
+        _check(offsets is not None, f"Must pass offsets for 2D input {what}.")
+        _check(offsets.dtype == torch.int32, "offsets must be int32.")
+        _check(offsets.is_cuda and offsets.is_contiguous() and offsets.dim() == 1, "offsets must be a 1-D contiguous GPU tensor")
+        return offsets.shape[0]
+
+    if XQ.dim() == 2 and WQ.dim() == 3:
+        G = need_offsets("XQ")
+        M, N, K = XQ.shape[0], WQ.shape[1], WQ.shape[2]
+        layout = _GROUPS_M_OFFSETS
+        _check(XQ.shape[1] == K and WQ.shape[0] == G, "XQ shape must be (total_M, K) and WQ shape must be (G, N, K).")
+        _check(x_scale.shape[0] == M, "x_scale shape must be (total_M).")
+        _check(w_scale.dim() == 2 and w_scale.shape[0] == G and w_scale.shape[1] == N, "w_scale shape must be (G, N).")
+        _check(output.dim() == 2 and output.shape[0] == M and output.shape[1] == N, "out shape must be (total_M, N).")
+    elif XQ.dim() == 3 and WQ.dim() == 2:
+        G = need_offsets("WQ")
+        M, N, K = XQ.shape[1], WQ.shape[0], WQ.shape[1]
+        layout = _GROUPS_N_OFFSETS
+        _check(XQ.shape[0] == G and XQ.shape[2] == K, "XQ shape must be (G, M, K) and WQ shape must be (total_N, K).")
+        _check(x_scale.dim() == 2 and x_scale.shape[0] == G and x_scale.shape[1] == M, "x_scale shape must be (G, M).")
+        _check(w_scale.shape[0] == N, "w_scale shape must be (total_N).")
+        _check(output.dim() == 2 and output.shape[0] == M and output.shape[1] == N, "out shape must be (M, total_N).")
+    elif XQ.dim() == 3 and WQ.dim() == 3:
+        _check(offsets is None, "Offsets should not be passed for 3D-3D inputs.")
+        G, M, K = XQ.shape
+        N = WQ.shape[1]
+        layout = _GROUPS_UNIFORM
+        _check(WQ.shape[0] == G and WQ.shape[2] == K, "XQ shape must be (G, M, K) and WQ shape must be (G, N, K).")
+        _check(x_scale.dim() == 2 and x_scale.shape[0] == G and x_scale.shape[1] == M, "x_scale shape must be (G, M).")
+        _check(w_scale.dim() == 2 and w_scale.shape[0] == G and w_scale.shape[1] == N, "w_scale shape must be (G, N).")
+        _check(output.dim() == 3 and tuple(output.shape) == (G, M, N), "out shape must be (G, M, N).")
+    elif XQ.dim() == 2 and WQ.dim() == 2:
+        G = need_offsets("s XQ and WQ")
+        M, N, K = XQ.shape[0], WQ.shape[0], XQ.shape[1]
+        layout = _GROUPS_K_OFFSETS
+        _check(WQ.shape[1] == K, "XQ shape must be (M, total_K) and WQ shape must be (N, total_K).")
+        _check(x_scale.shape[0] == G * M, "x_scale shape must be (G * M).")
+        _check(w_scale.shape[0] == G * N, "w_scale shape must be (G * N).")
+        _check(output.dim() == 3 and tuple(output.shape) == (G, M, N), "out shape must be (G, M, N).")
+    else:
+        _check(False, "Invalid input shapes. Must be one of 2D-2D, 3D-3D, 2D-3D, 3D-2D.")
+    if layout != _GROUPS_N_OFFSETS:
+        _check(N % 8 == 0, "N must be divisible by 8.")
+    _check(output.dtype == torch.bfloat16 and output.is_cuda and output.is_contiguous() and output.device == XQ.device,
+           "output must be a contiguous bfloat16 GPU tensor on the device of XQ")
+    _check(WQ.device == XQ.device and x_scale.device == XQ.device and w_scale.device == XQ.device and
+           (offsets is None or offsets.device == XQ.device), "all operands must be on the same device")
+    if output.numel() == 0:
+        return output
+    with _on_device(XQ.device):
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped_mm(
+            XQ.data_ptr(), WQ.data_ptr(), x_scale.data_ptr(), w_scale.data_ptr(),
+            None if offsets is None else offsets.data_ptr(), layout, G, M, N, K, output.data_ptr(),
+            _stream_ptr(XQ.device)))
+    return output
+
+
+def f8f8bf16_rowwise_batched(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True, output=None) -> torch.Tensor:
+    """XQ [B, M, K], WQ [B, N, K], x_scale [B, M], w_scale [B, N] -> bf16 [B, M, N]
+    (fp8_rowwise_batched_gemm.hip:199-254).  `bias` [B, N] (fp32 or bf16) is added per batch as the
+    reference's CUTLASS build does (f8f8bf16_rowwise_batched_common.cuh:272-275); its ROCm build
+    accepts the argument and drops it."""
+    _check(XQ.dim() == 3 and WQ.dim() == 3, "Inputs must have 3 dimensions, with the first being batch.")
+    _check(XQ.dtype == WQ.dtype, f"XQ and WQ dtypes must match, got {XQ.dtype} vs {WQ.dtype}")
+    _check(XQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ.dtype}")
+    _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
+    _check(use_fast_accum, "AMD does not support disabling use_fast_accum.")
+    _check(XQ.is_cuda and XQ.is_contiguous(), "XQ must be a contiguous GPU tensor")
+    _check(WQ.is_cuda and WQ.is_contiguous(), "WQ must be a contiguous GPU tensor")
+    B, M, K = XQ.shape
+    N = WQ.shape[1]
+    _check(WQ.shape[0] == B and WQ.shape[2] == K, "XQ must be (B, M, K) and WQ (B, N, K)")
+    _check(x_scale.numel() == B * M and w_scale.numel() == B * N, "scale sizes must match B*M and B*N")
+    _check(WQ.device == XQ.device and x_scale.device == XQ.device and w_scale.device == XQ.device,
+           "all operands must be on the same device")
+    if output is not None:
+        Y = output
+        _check(Y.dim() == 3, "Output tensor must have three dimensions.")
+        _check(tuple(Y.shape) == (B, M, N), "output has the wrong shape")
+        _check(Y.dtype == torch.bfloat16, "output must be bfloat16")
+        _check(Y.is_cuda and Y.is_contiguous() and Y.device == XQ.device, "output must be a contiguous GPU tensor")
+    else:
+        Y = torch.empty((B, M, N), dtype=torch.bfloat16, device=XQ.device)
+    if Y.numel() == 0:
+        return Y
+    xs, ws = x_scale.contiguous(), w_scale.contiguous()
+    bias_ptr, bias_code, _keep = _bias_args(bias, B * N, XQ.device)
+    with _on_device(XQ.device):
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_batched(
+            XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, B, M, N, K,
+            Y.data_ptr(), _stream_ptr(XQ.device)))
+    return Y
+
+
 # ---------------------------------------------------------------------------------------------
 # registration
 # ---------------------------------------------------------------------------------------------
@@ -220,6 +337,8 @@ _IMPLS = {
     "f8f8bf16_rowwise_grouped": f8f8bf16_rowwise_grouped,
     "f8f8bf16_rowwise_grouped_cat": f8f8bf16_rowwise_grouped_cat,
     "f8f8bf16_rowwise_grouped_stacked": f8f8bf16_rowwise_grouped_stacked,
+    "f8f8bf16_rowwise_grouped_mm": f8f8bf16_rowwise_grouped_mm,
+    "f8f8bf16_rowwise_batched": f8f8bf16_rowwise_batched,
 }
 
 
@@ -245,12 +364,25 @@ def _fake_grouped_stacked(XQ, WQ, x_scale, w_scale, M_sizes):
     return torch.empty((XQ.shape[0], WQ.shape[1]), dtype=torch.bfloat16, device=XQ.device)
 
 
+def _fake_grouped_mm(XQ, WQ, x_scale, w_scale, offsets, output):
+    return output
+
+
+def _fake_batched(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True, output=None):
+    # mslk/gemm/_meta.py:68-83
+    if output is not None:
+        return output
+    return torch.empty((XQ.shape[0], XQ.shape[1], WQ.shape[1]), dtype=torch.bfloat16, device=XQ.device)
+
+
 _FAKES = {
     "f8f8bf16_rowwise": _fake_rowwise,
     "f8f8bf16_rowwise_out": _fake_rowwise_out,
     "f8f8bf16_rowwise_grouped": _fake_grouped,
     "f8f8bf16_rowwise_grouped_cat": _fake_grouped_cat,
     "f8f8bf16_rowwise_grouped_stacked": _fake_grouped_stacked,
+    "f8f8bf16_rowwise_grouped_mm": _fake_grouped_mm,
+    "f8f8bf16_rowwise_batched": _fake_batched,
 }
 
 

@@ -40,6 +40,13 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 0, None, -1, 4, 4, None, 0, None) != 0
     assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 2, None, 4, 4, 4, None, 0, None) != 0
     assert b"bias" in L.mslk_amd_last_error()
+    assert L.mslk_amd_f8f8bf16_rowwise_grouped_mm(None, None, None, None, None, 9, 1, 4, 8, 16, None, None) != 0
+    assert b"layout" in L.mslk_amd_last_error()
+    assert L.mslk_amd_f8f8bf16_rowwise_grouped_mm(None, None, None, None, None, 1, 1, 4, 8, 16, None, None) != 0
+    assert b"offsets are required" in L.mslk_amd_last_error()
+    assert L.mslk_amd_f8f8bf16_rowwise_batched(None, None, None, None, None, 1, 2, 4, 8, 16, None, None) != 0
+    assert b"bias" in L.mslk_amd_last_error()
+    assert L.mslk_amd_f8f8bf16_rowwise_batched(None, None, None, None, None, 0, 0, 4, 8, 16, None, None) == 0
     # empty problems are a successful no-op and touch no pointer
     assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 0, None, 0, 4, 4, None, 0, None) == 0
     assert L.mslk_amd_quantize_fp8_row(None, 0, 0, 16, 16, None, 16, None, None, None) == 0
@@ -55,6 +62,12 @@ def test_ops_registered_with_reference_schemas():
     assert s == "mslk::f8f8bf16_rowwise_grouped(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor[]"
     s = str(torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked.default._schema)
     assert s.endswith("(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor M_sizes) -> Tensor")
+    s = str(torch.ops.mslk.f8f8bf16_rowwise_grouped_mm.default._schema)
+    assert s == ("mslk::f8f8bf16_rowwise_grouped_mm(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
+                 "Tensor? offsets, Tensor(a!) output) -> Tensor")
+    s = str(torch.ops.mslk.f8f8bf16_rowwise_batched.default._schema)
+    assert s == ("mslk::f8f8bf16_rowwise_batched(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
+                 "Tensor? bias=None, bool use_fast_accum=True, Tensor(a!)? output=None) -> Tensor")
     assert hasattr(torch.ops.mslk, "quantize_fp8_row")
 
 
@@ -78,6 +91,15 @@ def test_fake_kernels_give_reference_shapes():
             torch.empty(40, 512, dtype=F8, device=dev), torch.empty(4, 768, 512, dtype=F8, device=dev),
             torch.empty(40, device=dev), torch.empty(4, 768, device=dev), torch.empty(4, dtype=torch.int64, device=dev))
         assert y.shape == (40, 768)
+        out = torch.empty(40, 768, dtype=torch.bfloat16, device=dev)
+        y = torch.ops.mslk.f8f8bf16_rowwise_grouped_mm(
+            torch.empty(40, 512, dtype=F8, device=dev), torch.empty(4, 768, 512, dtype=F8, device=dev),
+            torch.empty(40, device=dev), torch.empty(4, 768, device=dev), torch.empty(4, dtype=torch.int32, device=dev), out)
+        assert y.shape == (40, 768)
+        y = torch.ops.mslk.f8f8bf16_rowwise_batched(
+            torch.empty(3, 40, 512, dtype=F8, device=dev), torch.empty(3, 768, 512, dtype=F8, device=dev),
+            torch.empty(3, 40, device=dev), torch.empty(3, 768, device=dev))
+        assert y.shape == (3, 40, 768) and y.dtype == torch.bfloat16
         q, s = torch.ops.mslk.quantize_fp8_row(torch.empty(2, 3, 100, dtype=torch.bfloat16, device=dev), None, 16)
         assert q.shape == (2, 3, 112) and q.dtype == F8 and s.shape == (2, 3) and s.dtype == torch.float32
 

@@ -80,7 +80,8 @@ def test_grouped_rejects_small_n_k_like_the_reference():
         torch.ops.mslk.f8f8bf16_rowwise_grouped(_dev(xq), _dev(wq), _dev(xs), _dev(ws))
 
 
-@pytest.mark.parametrize("ms,N,K", [([64, 0, 300, 5], 512, 512), ([1] * 16, 768, 1024), ([0, 0, 0, 700], 520, 272)])
+@pytest.mark.parametrize("ms,N,K", [([64, 0, 300, 5], 512, 512), ([1] * 16, 768, 1024), ([0, 0, 0, 700], 520, 272),
+                                    ([9, 40], 136, 200)])   # K not a multiple of 16: scalar tile path
 def test_stacked_grouped(ms, N, K):
     g = torch.Generator().manual_seed(33)
     xq, wq, xs, ws = _make_groups(ms, N, K, g)
