@@ -247,6 +247,20 @@ def main():
         q_bytes = 3.0 * M * K + 4.0 * M
         extras["quantize_cfg1"] = {"ms": q_ms, "GBps": q_bytes / (q_ms * 1e-3) / 1e9,
                                    "frac_hbm": q_bytes / (q_ms * 1e-3) / PEAK_HBM_BPS, "bytes": q_bytes}
+        # dequantize_fp8_row on the same shape: 1 B in + 2 B out per element, rotating over 10 code sets
+        qsets = [torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn) for _ in range(10)]
+        dq_out = [torch.empty(M, K, dtype=torch.bfloat16, device=dev) for _ in range(4)]
+
+        def dequant_step(i):
+            api.check(api.L.mslk_amd_dequantize_fp8_row(qsets[i % 10].data_ptr(), xs_tmp.data_ptr(), M, K,
+                                                        dq_out[i % 4].data_ptr(), api.stream))
+
+        for i in range(10):
+            dequant_step(i)
+        d_ms = _median_events_ms(dequant_step, 50)
+        extras["dequantize_cfg1"] = {"ms": d_ms, "GBps": q_bytes / (d_ms * 1e-3) / 1e9,
+                                     "frac_hbm": q_bytes / (d_ms * 1e-3) / PEAK_HBM_BPS, "bytes": q_bytes}
+        del qsets, dq_out
         if args.only == "quantize":
             print(json.dumps(extras))
             return

@@ -53,6 +53,29 @@ int mslk_amd_quantize_fp8_row(const void* x, int x_dtype, int64_t rows, int64_t 
                               void* xq, int64_t K_out, float* scale, const float* scale_ub, void* stream);
 
 /*
+ * The same quantizer over jagged groups of rows.  Replaces quantize_fp8_row(..., zero_start_index_M=...)
+ * (reference: mslk/quantize/triton/fp8_quantize.py:238-243 for the grouping, 123-129 for the row rule):
+ * the rows form rows / rows_per_group consecutive blocks; in block b only the first
+ * zero_start_index[b] rows hold data.  The remaining rows are never read and quantize exactly like
+ * all-zero rows (zero codes, the scale of a zero row).
+ *   zero_start_index  [rows / rows_per_group] int64 or int32 (index_dtype) in device memory
+ */
+#define MSLK_AMD_INDEX_I64 0
+#define MSLK_AMD_INDEX_I32 1
+int mslk_amd_quantize_fp8_row_jagged(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t x_row_stride,
+                                     void* xq, int64_t K_out, float* scale, const float* scale_ub,
+                                     const void* zero_start_index, int index_dtype, int64_t rows_per_group,
+                                     void* stream);
+
+/*
+ * Row-wise dequantization to bf16.  Replaces dequantize_fp8_row
+ * (reference: mslk/quantize/triton/fp8_quantize.py:1060-1113 kernel, 1140-1182 wrapper):
+ *   out[r, k] = bf16_rne( fl32( f32(xq[r, k]) * scale[r] ) )
+ *   xq [rows, K] e4m3fn contiguous, scale [rows] fp32, out [rows, K] bf16 contiguous.
+ */
+int mslk_amd_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out, void* stream);
+
+/*
  * Dense rowwise-scaled FP8 GEMM.  Replaces mslk::gemm::f8f8bf16_rowwise / f8f8bf16_rowwise_out
  * (reference: csrc/gemm/gemm_ops.cpp:31-34; host wrapper csrc/gemm/ck/fp8_rowwise/fp8fp8bf16_rowwise_gemm.hip:499-576;
  * math csrc/gemm/ck/fp8_rowwise/kernels/fp8_rowwise_common.h:54-82,168-204; bias semantics

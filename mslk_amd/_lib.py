@@ -20,6 +20,9 @@ SIGNATURES = {
     "mslk_amd_last_error": (c_char_p, []),
     "mslk_amd_quantize_fp8_row": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64,
                                           c_void_p, c_void_p, c_void_p]),
+    "mslk_amd_quantize_fp8_row_jagged": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64,
+                                                 c_void_p, c_void_p, c_void_p, c_int, c_int64, c_void_p]),
+    "mslk_amd_dequantize_fp8_row": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),

@@ -44,9 +44,37 @@ int mslk_amd_quantize_fp8_row(const void* x, int x_dtype, int64_t rows, int64_t 
   if (rows == 0) return 0;
   if (rows > kIntMax) return fail("quantize_fp8_row: rows (%lld) exceeds 2^31-1", (long long)rows);
   if (!x || !xq || !scale) return fail("quantize_fp8_row: null pointer");
-  return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub,
+  return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub, nullptr, 0, 1,
                                            (hipStream_t)stream),
                    "quantize_fp8_row launch");
+}
+
+int mslk_amd_quantize_fp8_row_jagged(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t x_row_stride,
+                                     void* xq, int64_t K_out, float* scale, const float* scale_ub,
+                                     const void* zero_start_index, int index_dtype, int64_t rows_per_group,
+                                     void* stream) {
+  if (x_dtype < 0 || x_dtype > 2) return fail("quantize_fp8_row_jagged: unsupported input dtype code %d", x_dtype);
+  if (index_dtype != MSLK_AMD_INDEX_I64 && index_dtype != MSLK_AMD_INDEX_I32)
+    return fail("quantize_fp8_row_jagged: unsupported index dtype code %d", index_dtype);
+  if (rows < 0 || K <= 0) return fail("quantize_fp8_row_jagged: rows must be >= 0 and K > 0 (got %lld, %lld)", (long long)rows, (long long)K);
+  if (K_out < K) return fail("quantize_fp8_row_jagged: K_out (%lld) < K (%lld)", (long long)K_out, (long long)K);
+  if (rows_per_group <= 0 || rows % rows_per_group != 0)
+    return fail("quantize_fp8_row_jagged: rows (%lld) must be a multiple of rows_per_group (%lld)", (long long)rows,
+                (long long)rows_per_group);
+  if (rows == 0) return 0;
+  if (rows > kIntMax) return fail("quantize_fp8_row_jagged: rows (%lld) exceeds 2^31-1", (long long)rows);
+  if (!x || !xq || !scale || !zero_start_index) return fail("quantize_fp8_row_jagged: null pointer");
+  return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub,
+                                           zero_start_index, index_dtype == MSLK_AMD_INDEX_I32, rows_per_group,
+                                           (hipStream_t)stream),
+                   "quantize_fp8_row_jagged launch");
+}
+
+int mslk_amd_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out, void* stream) {
+  if (rows < 0 || K < 0) return fail("dequantize_fp8_row: negative dimension");
+  if (rows == 0 || K == 0) return 0;
+  if (!xq || !scale || !out) return fail("dequantize_fp8_row: null pointer");
+  return check_hip(launch_dequantize_fp8_row(xq, scale, rows, K, out, (hipStream_t)stream), "dequantize_fp8_row launch");
 }
 
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }

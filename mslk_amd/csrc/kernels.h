@@ -6,8 +6,13 @@
 
 namespace mslk_amd {
 
+// zero_start != nullptr: jagged rows (blocks of rows_per_group rows, the first zero_start[block] are live).
 hipError_t launch_quantize_fp8_row(const void* x, int dtype, int64_t rows, int64_t K, int64_t in_stride,
-                                   void* xq, int64_t K_out, float* scale, const float* scale_ub, hipStream_t s);
+                                   void* xq, int64_t K_out, float* scale, const float* scale_ub,
+                                   const void* zero_start, int zero_start_is_i32, int64_t rows_per_group,
+                                   hipStream_t s);
+hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out,
+                                     hipStream_t s);
 hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t s);
 
 // One GEMM problem: Y[M,N] = bf16(XQ[M,K] . WQ[N,K]^T * xs[:,None] * ws[None,:] + bias[None,:]).

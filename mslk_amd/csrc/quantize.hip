@@ -134,6 +134,23 @@ MSLK_AMD_DEVINL void scales_from_amax(float amax, const float* scale_ub, float& 
   scale = 1.0f / inv;
 }
 
+// Jagged rows (reference: JAGGED branch of _kernel_quantize_fp8_row, fp8_quantize.py:123-129): rows are
+// grouped in blocks of `rows_per_group`; inside block b only the first zero_start[b] rows hold data,
+// the others are treated as all-zero rows and are never read.
+struct JaggedRows {
+  const void* zero_start;   // nullptr: every row is live
+  int64_t rows_per_group;
+  int index_is_i32;
+};
+
+MSLK_AMD_DEVINL bool row_is_live(const JaggedRows& j, int64_t row) {
+  if (j.zero_start == nullptr) return true;
+  const int64_t b = row / j.rows_per_group, n = row - b * j.rows_per_group;
+  const int64_t live = j.index_is_i32 ? (int64_t) static_cast<const int32_t*>(j.zero_start)[b]
+                                      : static_cast<const int64_t*>(j.zero_start)[b];
+  return n < live;
+}
+
 template <int TEAM>
 MSLK_AMD_DEVINL uint32_t team_max(uint32_t m, uint32_t* smem, int team_in_block) {
 #pragma unroll
@@ -155,7 +172,7 @@ MSLK_AMD_DEVINL uint32_t team_max(uint32_t m, uint32_t* smem, int team_in_block)
 template <int DTYPE, int TEAM, int NV, bool CACHED>
 __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
     const void* __restrict__ x, int64_t rows, int K, int64_t in_stride, uint8_t* __restrict__ out,
-    int64_t out_stride, float* __restrict__ scale, const float* __restrict__ scale_ub) {
+    int64_t out_stride, float* __restrict__ scale, const float* __restrict__ scale_ub, JaggedRows jag) {
   constexpr int TEAMS = 256 / TEAM;
   constexpr int ELEM_BYTES = (DTYPE == 2) ? 4 : 2;
   __shared__ uint32_t smem[4];
@@ -163,6 +180,7 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
   const int lane = threadIdx.x % TEAM;
   const int64_t row = (int64_t)blockIdx.x * TEAMS + team_in_block;
   const bool valid = row < rows;
+  const bool live = valid && row_is_live(jag, row);   // uniform over the team
   const int nvec = K >> 3;
   const char* row_ptr = reinterpret_cast<const char*>(x) + (valid ? row : 0) * in_stride * ELEM_BYTES;
 
@@ -172,13 +190,13 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = i * TEAM + lane;
-      if (valid && idx < nvec) {
+      if (live && idx < nvec) {
         cache[i] = load_vec8<DTYPE>(row_ptr, idx);
         m = absmax_bits<DTYPE>(m, cache[i]);
       }
     }
   } else {
-    if (valid)
+    if (live)
       for (int idx = lane; idx < nvec; idx += TEAM) m = absmax_bits<DTYPE>(m, load_vec8<DTYPE>(row_ptr, idx));
   }
   m = team_max<TEAM>(finish_absmax_bits<DTYPE>(m), smem, team_in_block);
@@ -189,7 +207,9 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
   if (lane == 0) scale[row] = sc;
 
   uint2* out_row = reinterpret_cast<uint2*>(out + row * out_stride);
-  if constexpr (CACHED) {
+  if (!live) {   // an empty row quantizes to zero codes
+    for (int idx = lane; idx < nvec; idx += TEAM) store8_stream(out_row + idx, make_uint2(0u, 0u));
+  } else if constexpr (CACHED) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = i * TEAM + lane;
@@ -207,11 +227,12 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
 template <int DTYPE>
 __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
     const void* __restrict__ x, int64_t rows, int64_t K, int64_t in_stride, uint8_t* __restrict__ out,
-    int64_t out_stride, float* __restrict__ scale, const float* __restrict__ scale_ub) {
+    int64_t out_stride, float* __restrict__ scale, const float* __restrict__ scale_ub, JaggedRows jag) {
   using elem_t = typename Traits<DTYPE>::elem_t;
   __shared__ uint32_t smem[4];
   const int64_t row = blockIdx.x;
   const elem_t* xr = reinterpret_cast<const elem_t*>(x) + row * in_stride;
+  if (!row_is_live(jag, row)) K = 0;   // nothing of the row is read; all codes become zero
   uint32_t m = 0;
   for (int64_t k = threadIdx.x; k < K; k += 256) {
     if constexpr (DTYPE == 2) m = max(m, __float_as_uint(xr[k]) & 0x7FFFFFFFu);
@@ -233,6 +254,39 @@ __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
   }
 }
 
+// Row-wise dequantization (reference: _kernel_dequantize_fp8_row, fp8_quantize.py:1060-1113):
+// out = bf16_rne(fl32(fp8 -> f32) * scale[row]).  1 byte in, 2 bytes out per element: HBM-bound.
+// A lane converts 16 consecutive codes of one row (K % 16 == 0) per iteration.
+__global__ __launch_bounds__(256) void dequantize_rows_vec_kernel(const uint8_t* __restrict__ xq,
+                                                                  const float* __restrict__ scale, int64_t chunks,
+                                                                  int chunks_per_row, uint16_t* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += stride) {
+    const v4i q = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(xq) + c);
+    const float sc = scale[c / chunks_per_row];
+    const int w[4] = {q.x, q.y, q.z, q.w};
+    uint32_t o[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[i], false);
+      const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[i], true);
+      o[2 * i] = pack_bf16x2(lo[0] * sc, lo[1] * sc);
+      o[2 * i + 1] = pack_bf16x2(hi[0] * sc, hi[1] * sc);
+    }
+    v4i* dst = reinterpret_cast<v4i*>(out) + 2 * c;
+    __builtin_nontemporal_store(v4i{(int)o[0], (int)o[1], (int)o[2], (int)o[3]}, dst);
+    __builtin_nontemporal_store(v4i{(int)o[4], (int)o[5], (int)o[6], (int)o[7]}, dst + 1);
+  }
+}
+
+__global__ __launch_bounds__(256) void dequantize_rows_generic_kernel(const uint8_t* __restrict__ xq,
+                                                                      const float* __restrict__ scale, int64_t total,
+                                                                      int64_t K, uint16_t* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+    out[i] = (uint16_t)f32_to_bf16_bits(__builtin_amdgcn_cvt_f32_fp8((int)xq[i], 0) * scale[i / K]);
+}
+
 __global__ void cast_e4m3fn_kernel(const float* __restrict__ in, int64_t n, uint8_t* __restrict__ out) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
@@ -241,7 +295,8 @@ __global__ void cast_e4m3fn_kernel(const float* __restrict__ in, int64_t n, uint
 
 template <int DTYPE>
 hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_stride, uint8_t* out,
-                             int64_t out_stride, float* scale, const float* scale_ub, hipStream_t s) {
+                             int64_t out_stride, float* scale, const float* scale_ub, JaggedRows jag,
+                             hipStream_t s) {
   constexpr int ELEM_BYTES = (DTYPE == 2) ? 4 : 2;
   constexpr int NV = 16;
   const bool vec_ok = (K % 8 == 0) && (K < (int64_t(1) << 31)) && ((in_stride * ELEM_BYTES) % 16 == 0) &&
@@ -249,7 +304,7 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
                       (reinterpret_cast<uintptr_t>(out) % 8 == 0);
   if (!vec_ok) {
     quantize_rows_generic_kernel<DTYPE><<<dim3((unsigned)rows), dim3(256), 0, s>>>(
-        x, rows, K, in_stride, out, out_stride, scale, scale_ub);
+        x, rows, K, in_stride, out, out_stride, scale, scale_ub, jag);
     return hipGetLastError();
   }
   const int k = (int)K;
@@ -257,17 +312,17 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
   if (K <= kWave * 8 * NV && rows >= 2048) {
     const unsigned blocks = (unsigned)((rows + 3) / 4);
     if (K <= kWave * 8 * 4)
-      quantize_rows_vec_kernel<DTYPE, 64, 4, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub);
+      quantize_rows_vec_kernel<DTYPE, 64, 4, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
     else if (K <= kWave * 8 * 8)
-      quantize_rows_vec_kernel<DTYPE, 64, 8, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub);
+      quantize_rows_vec_kernel<DTYPE, 64, 8, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
     else
-      quantize_rows_vec_kernel<DTYPE, 64, NV, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub);
+      quantize_rows_vec_kernel<DTYPE, 64, NV, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else if (K <= 256 * 8 * 4) {
-    quantize_rows_vec_kernel<DTYPE, 256, 4, true><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub);
+    quantize_rows_vec_kernel<DTYPE, 256, 4, true><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else if (K <= 256 * 8 * NV) {
-    quantize_rows_vec_kernel<DTYPE, 256, NV, true><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub);
+    quantize_rows_vec_kernel<DTYPE, 256, NV, true><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else {
-    quantize_rows_vec_kernel<DTYPE, 256, 1, false><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub);
+    quantize_rows_vec_kernel<DTYPE, 256, 1, false><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   }
   return hipGetLastError();
 }
@@ -276,13 +331,36 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
 
 hipError_t launch_quantize_fp8_row(const void* x, int dtype, int64_t rows, int64_t K, int64_t in_stride,
                                    void* xq, int64_t K_out, float* scale, const float* scale_ub,
+                                   const void* zero_start, int zero_start_is_i32, int64_t rows_per_group,
                                    hipStream_t s) {
   uint8_t* out = reinterpret_cast<uint8_t*>(xq);
+  const JaggedRows jag{zero_start, rows_per_group > 0 ? rows_per_group : 1, zero_start_is_i32};
   switch (dtype) {
-    case 0: return launch_quantize_t<0>(x, rows, K, in_stride, out, K_out, scale, scale_ub, s);
-    case 1: return launch_quantize_t<1>(x, rows, K, in_stride, out, K_out, scale, scale_ub, s);
-    default: return launch_quantize_t<2>(x, rows, K, in_stride, out, K_out, scale, scale_ub, s);
+    case 0: return launch_quantize_t<0>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+    case 1: return launch_quantize_t<1>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+    default: return launch_quantize_t<2>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
   }
+}
+
+hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out,
+                                     hipStream_t s) {
+  const int64_t total = rows * K;
+  if (total <= 0) return hipSuccess;
+  const bool vec_ok = K % 16 == 0 && reinterpret_cast<uintptr_t>(xq) % 16 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0;
+  if (vec_ok) {
+    const int64_t chunks = total / 16;
+    const int64_t want = (chunks + 255) / 256;
+    // enough resident waves to cover HBM latency; each lane then walks the tensor grid-stride
+    const unsigned blocks = (unsigned)(want > 256 * 32 ? 256 * 32 : want);
+    dequantize_rows_vec_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const uint8_t*>(xq), scale, chunks, (int)(K / 16),
+                                                     reinterpret_cast<uint16_t*>(out));
+  } else {
+    const int64_t want = (total + 255) / 256;
+    const unsigned blocks = (unsigned)(want > 65536 ? 65536 : want);
+    dequantize_rows_generic_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const uint8_t*>(xq), scale, total, K,
+                                                         reinterpret_cast<uint16_t*>(out));
+  }
+  return hipGetLastError();
 }
 
 hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t s) {

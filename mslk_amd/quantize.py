@@ -37,8 +37,8 @@ class _on_device:
             self.ctx.__exit__(*exc)
 
 
-def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, align_rows_to: Optional[int] = None
-                   ) -> Tuple[torch.Tensor, torch.Tensor]:
+def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, align_rows_to: Optional[int] = None,
+                   zero_start_index_M: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     if a.dtype not in _DTYPE_CODE:
         raise RuntimeError(f"quantize_fp8_row: unsupported input dtype {a.dtype} (bf16, fp16, fp32 are supported)")
     if a.dim() < 1:
@@ -69,6 +69,25 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
     if scale_ub is not None:
         scale_ub = scale_ub.to(device=a.device, dtype=torch.float32).reshape(-1)[:1].contiguous()
         ub_ptr = scale_ub.data_ptr()
+    if zero_start_index_M is not None:
+        # One entry per [N, K] matrix of the input viewed as [B, M, N, K] (fp8_quantize.py:236-243).
+        rows_per_group = a.shape[-2] if a.dim() >= 2 else 1
+        zs = zero_start_index_M
+        if zs.device != a.device:
+            raise RuntimeError("'zero_start_index_M' must be on the same device as 'a'")
+        if zs.dtype not in (torch.int64, torch.int32):
+            raise RuntimeError(f"zero_start_index_M must be int64 or int32, got {zs.dtype}")
+        if rows_per_group == 0 or zs.numel() * rows_per_group != rows:
+            raise RuntimeError(f"zero_start_index_M must have one entry per group of {rows_per_group} rows "
+                               f"({rows // max(rows_per_group, 1)} entries), got {zs.numel()}")
+        zs = zs.contiguous()
+        if rows > 0:
+            with _on_device(a.device):
+                _lib.check(_lib.lib().mslk_amd_quantize_fp8_row_jagged(
+                    a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
+                    scale.data_ptr(), ub_ptr, zs.data_ptr(), 0 if zs.dtype == torch.int64 else 1, rows_per_group,
+                    _stream_ptr(a.device)))
+        return xq, scale
     if rows > 0:
         with _on_device(a.device):
             _lib.check(_lib.lib().mslk_amd_quantize_fp8_row(
@@ -77,7 +96,7 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
     return xq, scale
 
 
-def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None):
+def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None, zero_start_index_M=None):
     # shape function of the reference (fp8_quantize.py:381-407)
     K = a.shape[-1]
     if align_rows_to is not None:
@@ -89,7 +108,8 @@ def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None):
 # Registered with the low-level library API (a few microseconds of dispatch per call); GPU kernel only.
 _library = torch.library.Library("mslk", "FRAGMENT")
 if not hasattr(torch.ops.mslk, "quantize_fp8_row"):
-    _library.define("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, int? align_rows_to=None) -> (Tensor, Tensor)")
+    _library.define("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, int? align_rows_to=None, "
+                    "Tensor? zero_start_index_M=None) -> (Tensor, Tensor)")
     _library.impl("quantize_fp8_row", _quantize_impl, "CUDA")
     torch.library.register_fake("mslk::quantize_fp8_row", _quantize_fp8_row_fake, lib=_library)
 
@@ -109,17 +129,54 @@ def quantize_fp8_row(
     The numerics are those of the reference's torch branch (the contract this build is checked
     against bit for bit): amax is clamped at 1e-12 in the input dtype, so `eps_opt` -- which only the
     reference's Triton branch reads -- has no effect; `use_triton` is accepted and ignored (there is one
-    implementation).  `zero_start_index_M` (jagged rows) is not supported and raises.
+    implementation).  With `zero_start_index_M` (one entry per [N, K] matrix of the input viewed as
+    [B, M, N, K]) the rows n >= zero_start_index_M[b, m] are not read and quantize like all-zero rows
+    (fp8_quantize.py:123-129).
     The input must live on a GPU: there is no CPU implementation in this package.
     """
     if not a.is_cuda:
         raise RuntimeError("mslk_amd.quantize_fp8_row: input must be a GPU tensor (no CPU implementation)")
-    if zero_start_index_M is not None:
-        raise NotImplementedError("mslk_amd.quantize_fp8_row: zero_start_index_M (jagged rows) is not supported")
-    a_fp8, a_scale = torch.ops.mslk.quantize_fp8_row(a, scale_ub, align_rows_to)
+    a_fp8, a_scale = torch.ops.mslk.quantize_fp8_row(a, scale_ub, align_rows_to, zero_start_index_M)
     if output_device is not None and torch.device(output_device) != a.device:
         a_fp8, a_scale = a_fp8.to(output_device), a_scale.to(output_device)
     return a_fp8, a_scale
+
+
+def _dequantize_impl(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
+    if not (xq.is_contiguous() and x_scale.is_contiguous()):
+        raise RuntimeError("Input tensors must be contiguous")
+    if xq.dtype != FP8_DTYPE:
+        raise RuntimeError(f"dequantize_fp8_row: xq must be {FP8_DTYPE}, got {xq.dtype}")
+    if x_scale.dtype != torch.float32 or x_scale.device != xq.device:
+        raise RuntimeError("dequantize_fp8_row: x_scale must be a float32 tensor on the device of xq")
+    if xq.dim() < 1:
+        raise RuntimeError("dequantize_fp8_row: xq must have at least one dimension")
+    K = xq.shape[-1]
+    rows = xq.numel() // K if K else 0
+    if x_scale.numel() != (rows if K else x_scale.numel()):
+        raise RuntimeError(f"dequantize_fp8_row: x_scale must have one entry per row ({rows}), got {x_scale.numel()}")
+    out = torch.empty(xq.shape, dtype=torch.bfloat16, device=xq.device)
+    if rows > 0:
+        with _on_device(xq.device):
+            _lib.check(_lib.lib().mslk_amd_dequantize_fp8_row(xq.data_ptr(), x_scale.data_ptr(), rows, K, out.data_ptr(),
+                                                              _stream_ptr(xq.device)))
+    return out
+
+
+if not hasattr(torch.ops.mslk, "dequantize_fp8_row"):
+    _library.define("dequantize_fp8_row(Tensor xq, Tensor x_scale) -> Tensor")
+    _library.impl("dequantize_fp8_row", _dequantize_impl, "CUDA")
+    torch.library.register_fake(
+        "mslk::dequantize_fp8_row",
+        lambda xq, x_scale: torch.empty(xq.shape, dtype=torch.bfloat16, device=xq.device), lib=_library)
+
+
+def dequantize_fp8_row(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
+    """Row-wise dequantization to bf16 along the last axis (reference signature, fp8_quantize.py:1140-1182):
+    out = bf16(float(xq) * x_scale[..., None]), the product taken in fp32."""
+    if not xq.is_cuda:
+        raise RuntimeError("mslk_amd.dequantize_fp8_row: input must be a GPU tensor (no CPU implementation)")
+    return torch.ops.mslk.dequantize_fp8_row(xq, x_scale)
 
 
 def quantize_fp8_per_row(

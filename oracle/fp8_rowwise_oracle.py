@@ -59,6 +59,27 @@ def dequantize_fp8_row(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
     return xq.to(torch.float32) * x_scale.to(torch.float32).reshape(*xq.shape[:-1], 1)
 
 
+def dequantize_fp8_row_bf16(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
+    """What the reference's dequantize kernel stores (fp8_quantize.py:1096-1112): the fp32 product
+    of the decoded code and the row scale, rounded to bf16 (nearest even) by the store."""
+    return dequantize_fp8_row(xq, x_scale).to(torch.bfloat16)
+
+
+def quantize_fp8_row_jagged(a: torch.Tensor, zero_start_index_M: torch.Tensor,
+                            scale_ub: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Jagged variant (fp8_quantize.py:236-243 grouping, 123-129 row rule): with `a` viewed as
+    [B, M, N, K] and zero_start_index_M as [B, M], row n of matrix (b, m) is loaded with an empty
+    mask when n >= zero_start_index_M[b, m], i.e. it is quantized as a row of zeros."""
+    a4 = a
+    while a4.dim() < 4:
+        a4 = a4.unsqueeze(0)
+    zs = zero_start_index_M.reshape(a4.shape[0], a4.shape[1]).to(torch.int64)
+    n = torch.arange(a4.shape[2]).reshape(1, 1, -1)
+    live = n < zs[:, :, None]
+    masked = torch.where(live[..., None], a4, torch.zeros((), dtype=a.dtype)).reshape(a.shape)
+    return quantize_fp8_row(masked, scale_ub)
+
+
 def dequant_matmul(xq: torch.Tensor, wq: torch.Tensor, x_scale: torch.Tensor,
                    w_scale: torch.Tensor, bias: Optional[torch.Tensor] = None,
                    dtype: torch.dtype = torch.float32) -> torch.Tensor:

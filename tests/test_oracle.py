@@ -208,3 +208,52 @@ def test_golden_quantize_rows():
         for got_q, got_s in ((q.view(torch.uint8), s), (cq, cs)):
             assert torch.equal(got_q[~nan], want_q[~nan]), case["name"]
             assert torch.equal(got_s.view(torch.int32)[~nan], want_s[~nan]), case["name"]
+
+
+def test_jagged_rows_are_zero_rows_and_live_rows_are_untouched():
+    g = torch.Generator().manual_seed(77)
+    a = torch.randn(3, 5, 7, 24, generator=g).bfloat16()
+    zs = torch.randint(0, 8, (3, 5), generator=g)
+    q, s = O.quantize_fp8_row_jagged(a, zs)
+    q0, s0 = O.quantize_fp8_row(a)
+    zero_row_scale = O.quantize_fp8_row(torch.zeros(1, 24, dtype=torch.bfloat16))[1].item()
+    assert zero_row_scale == 2.236306529429413e-15   # 1 / fl32(fl32(1 / bf16(1e-12)) * 448)
+    for b in range(3):
+        for m in range(5):
+            k = int(zs[b, m])
+            assert torch.equal(q[b, m, :k].view(torch.uint8), q0[b, m, :k].view(torch.uint8))
+            assert torch.equal(s[b, m, :k], s0[b, m, :k])
+            assert (q[b, m, k:].view(torch.uint8) == 0).all()
+            assert (s[b, m, k:] == zero_row_scale).all()
+    # lower-rank inputs are grouped by their second-to-last dimension
+    a2 = torch.randn(20, 30, generator=g).bfloat16()
+    q, s = O.quantize_fp8_row_jagged(a2, torch.tensor([6]))
+    assert (q[6:].view(torch.uint8) == 0).all() and torch.equal(s[:6], O.quantize_fp8_row(a2)[1][:6])
+
+
+def test_dequantize_closed_forms():
+    codes = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).reshape(1, 256)
+    # scale 1: every finite e4m3fn value is exactly representable in bf16
+    d = O.dequantize_fp8_row_bf16(codes, torch.ones(1))
+    ref = codes.to(torch.float32)
+    ok = ~torch.isnan(ref)
+    assert torch.equal(d.float()[ok], ref[ok]) and torch.isnan(d.float()[~ok]).all()
+    # powers of two scale exactly; 448 * 2^-10 etc. stay normal in bf16
+    for e in (-10, -3, 4):
+        d = O.dequantize_fp8_row_bf16(codes, torch.tensor([2.0 ** e]))
+        assert torch.equal(d.float()[ok], ref[ok] * 2.0 ** e)
+    # roundings worked by hand (bf16 spacing in [1, 2) is 2^-7):
+    one = torch.tensor([[1.0]]).to(torch.float8_e4m3fn)
+    assert O.dequantize_fp8_row_bf16(one, torch.tensor([1.0 + 2.0 ** -8])).item() == 1.0            # tie -> even
+    assert O.dequantize_fp8_row_bf16(one, torch.tensor([1.0 + 3 * 2.0 ** -8])).item() == 1.015625   # tie -> even (up)
+    x175 = torch.tensor([[1.75]]).to(torch.float8_e4m3fn)
+    assert O.dequantize_fp8_row_bf16(x175, torch.tensor([1.0 + 2.0 ** -8])).item() == 1.7578125     # 1.7568359375 -> up
+    x15 = torch.tensor([[1.5]]).to(torch.float8_e4m3fn)
+    assert O.dequantize_fp8_row_bf16(x15, torch.tensor([1.0 + 2.0 ** -9])).item() == 1.5            # 1.5029296875 -> down
+    # round trip: e4m3fn keeps 3 mantissa bits, bf16 7
+    g = torch.Generator().manual_seed(3)
+    a = torch.randn(64, 256, generator=g).bfloat16()
+    q, sc = O.quantize_fp8_row(a)
+    back = O.dequantize_fp8_row_bf16(q, sc).float()
+    amax = a.float().abs().amax(dim=1, keepdim=True)
+    assert ((back - a.float()).abs() <= a.float().abs() * 2.0 ** -4 + amax * 2.0 ** -9).all()

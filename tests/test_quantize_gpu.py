@@ -130,8 +130,10 @@ def test_legacy_name_and_errors():
     a = torch.randn(8, 64).bfloat16()
     xq, s = mslk_amd.quantize_fp8_per_row(a.to(DEV))
     assert_quant_bit_exact(a, xq, s)
-    with pytest.raises(NotImplementedError):
-        mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=torch.zeros(8, device=DEV))
+    with pytest.raises(RuntimeError, match="one entry per group"):
+        mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=torch.zeros(8, dtype=torch.int64, device=DEV))
+    with pytest.raises(RuntimeError, match="int64 or int32"):
+        mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=torch.zeros(1, device=DEV))
     with pytest.raises(RuntimeError):
         mslk_amd.quantize_fp8_row(torch.zeros(4, 0, dtype=torch.bfloat16, device=DEV))
     xq, s = mslk_amd.quantize_fp8_row(torch.zeros(0, 64, dtype=torch.bfloat16, device=DEV))
@@ -149,3 +151,71 @@ def test_round_trip_and_full_size_properties():
     assert ((c & 0x7F) == 0x7E).any(dim=1).all()
     deq = xq.float().cpu() * s.cpu()[:, None]
     assert torch.allclose(deq, wl.x.float(), atol=2e-1, rtol=1e-1)  # the reference's own round-trip bound
+
+
+@pytest.mark.parametrize("shape,align,idx_dtype", [
+    ((20, 30), None, torch.int64), ((20, 30), 16, torch.int64), ((6, 4, 2, 3), None, torch.int64),
+    ((4, 2, 3), None, torch.int32), ((8, 40, 512), None, torch.int64), ((3, 2, 300, 1024), None, torch.int32),
+    ((2, 2500, 4096), None, torch.int64), ((5, 9, 20000), None, torch.int64), ((16, 64, 136), 128, torch.int64),
+])
+def test_jagged_rows(shape, align, idx_dtype):
+    """Shapes of test/quantize/triton/fp8_quantize_test.py:201-222 plus every kernel variant."""
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.randn(shape, generator=g).bfloat16()
+    groups = 1
+    for d in shape[:-2]:
+        groups *= d
+    zs = torch.randint(0, shape[-2] + 1, (groups,), generator=g).to(idx_dtype)
+    zs[0] = shape[-2]      # one full group
+    if groups > 1:
+        zs[-1] = 0         # one empty group
+    # poison the rows that must not be read: a NaN there would change the result if it were
+    poisoned = a.clone().view(groups, shape[-2], shape[-1])
+    for gi in range(groups):
+        poisoned[gi, int(zs[gi]):] = float("nan")
+    xq, s = mslk_amd.quantize_fp8_row(poisoned.view(shape).to(DEV), zero_start_index_M=zs.to(DEV), align_rows_to=align)
+    torch.cuda.synchronize()
+    rq, rs = O.quantize_fp8_row_jagged(a, zs)
+    K = shape[-1]
+    got = codes(xq)
+    if align is not None:
+        K_out = (K + align - 1) // align * align
+        assert got.shape[-1] == K_out and (got[..., K:] == 0).all()
+        got = got[..., :K]
+    assert torch.equal(got, codes(rq))
+    assert torch.equal(bits32(s), bits32(rs))
+    assert s.shape == a.shape[:-1]
+
+
+@pytest.mark.parametrize("shape", [(1, 256), (3, 16), (7, 777), (64, 1024), (2, 3, 17, 136), (2500, 4096), (5, 3)])
+def test_dequantize_bit_exact(shape):
+    g = torch.Generator().manual_seed(sum(shape))
+    rows = 1
+    for d in shape[:-1]:
+        rows *= d
+    q = torch.randint(0, 256, shape, generator=g, dtype=torch.uint8)
+    if shape == (1, 256):
+        q = torch.arange(256, dtype=torch.uint8).reshape(1, 256)    # every code, NaNs included
+    q = q.view(torch.float8_e4m3fn)
+    sc = torch.rand(shape[:-1], generator=g) * 4 + 2.0 ** -12
+    out = mslk_amd.dequantize_fp8_row(q.to(DEV), sc.to(DEV))
+    torch.cuda.synchronize()
+    ref = O.dequantize_fp8_row_bf16(q, sc)
+    assert out.shape == q.shape and out.dtype == torch.bfloat16
+    o16, r16 = out.cpu().view(torch.int16), ref.view(torch.int16)
+    nan = torch.isnan(ref.float())
+    assert torch.isnan(out.cpu().float()[nan]).all()
+    assert torch.equal(o16[~nan], r16[~nan])
+
+
+def test_dequantize_round_trip_full_size():
+    g = torch.Generator().manual_seed(12)
+    a = torch.randn(4096, 4096, generator=g).bfloat16().to(DEV)
+    xq, s = mslk_amd.quantize_fp8_row(a)
+    back = mslk_amd.dequantize_fp8_row(xq, s).float()
+    af = a.float()
+    assert ((back - af).abs() <= af.abs() * 2.0 ** -4 + af.abs().amax(dim=1, keepdim=True) * 2.0 ** -9).all()
+    # dequantize(quantize(.)) is idempotent: quantizing the result again reproduces codes and values
+    xq2, s2 = mslk_amd.quantize_fp8_row(back.bfloat16())
+    back2 = mslk_amd.dequantize_fp8_row(xq2, s2).float()
+    assert (back2 - back).abs().max() <= back.abs().max() * 2.0 ** -7
