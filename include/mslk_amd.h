@@ -91,6 +91,15 @@ int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_sca
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * The same GEMM with an fp16 (IEEE half, round to nearest even, overflow to infinity) output.
+ * Replaces mslk::gemm::f8f8f16_rowwise (reference: csrc/gemm/gemm_ops.cpp:88-89,
+ * csrc/gemm/ck/fp8_rowwise/fp8fp8fp16_rowwise_gemm.hip:66-133).  Arguments as above; y is fp16.
+ */
+int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                             const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                             void* stream);
+
+/*
  * Grouped (MoE) rowwise FP8 GEMM over G independent problems given as host arrays of device
  * pointers.  Replaces mslk::gemm::f8f8bf16_rowwise_grouped (TensorList API; reference:
  * csrc/gemm/gemm_ops.cpp:37-38, csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:481-559,586-593).
@@ -139,6 +148,19 @@ int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, co
 int mslk_amd_f8f8bf16_rowwise_grouped_mm(const void* xq, const void* wq, const float* x_scale,
                                          const float* w_scale, const int32_t* offsets_dev, int layout, int G,
                                          int64_t M, int64_t N, int64_t K, void* y, void* stream);
+
+/*
+ * Grouped GEMM over pre-padded groups: xq [G, M, K], wq [G, N, K], x_scale [G, M], w_scale [G, N],
+ * y [G, M, N]; only the first zero_start_index_M[g] (int64, device memory) rows of group g are
+ * multiplied.  With zeroing_output != 0 the whole of y is zero-filled first, so the padding rows read
+ * as zero; otherwise they are left untouched.  Replaces mslk::gemm::f8f8bf16_rowwise_grouped_dynamic
+ * (reference: csrc/gemm/gemm_ops.cpp:43-44, csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:656-714,
+ * which marks the operator deprecated in favour of the stacked / offsets entry points above).
+ */
+int mslk_amd_f8f8bf16_rowwise_grouped_dynamic(const void* xq, const void* wq, const float* x_scale,
+                                              const float* w_scale, const int64_t* zero_start_index_M_dev, int G,
+                                              int64_t M, int64_t N, int64_t K, void* y, int zeroing_output,
+                                              void* stream);
 
 /*
  * Batched rowwise FP8 GEMM: Y[b] = bf16(XQ[b] . WQ[b]^T * x_scale[b][:,None] * w_scale[b][None,:] + bias[b]).

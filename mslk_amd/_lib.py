@@ -25,6 +25,8 @@ SIGNATURES = {
     "mslk_amd_dequantize_fp8_row": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
+    "mslk_amd_f8f8f16_rowwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                         c_int64, c_int64, c_int64, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "mslk_amd_f8f8bf16_rowwise_grouped": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),
                                                   POINTER(c_void_p), POINTER(c_void_p), POINTER(c_int64),
@@ -33,6 +35,8 @@ SIGNATURES = {
                                                           c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise_grouped_mm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                                      c_int64, c_int64, c_int64, c_void_p, c_void_p]),
+    "mslk_amd_f8f8bf16_rowwise_grouped_dynamic": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                                          c_int64, c_int64, c_int64, c_void_p, c_int, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise_batched": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
                                                   c_int64, c_int64, c_int64, c_void_p, c_void_p]),
     "mslk_amd_debug_cast_e4m3fn": (c_int, [c_void_p, c_int64, c_void_p, c_void_p]),

@@ -79,23 +79,35 @@ int mslk_amd_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows
 
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
 
-int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
-                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
-                              void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
-  if (M < 0 || N < 0 || K < 0) return fail("f8f8bf16_rowwise: negative dimension");
-  if (M > kIntMax || N > kIntMax || K > kIntMax) return fail("f8f8bf16_rowwise: dimension exceeds 2^31-1");
-  if (bias_dtype < 0 || bias_dtype > 2) return fail("f8f8bf16_rowwise: bad bias dtype code %d", bias_dtype);
-  if ((bias_dtype != 0) != (bias != nullptr)) return fail("f8f8bf16_rowwise: bias pointer and bias dtype disagree");
+static int rowwise_impl(const char* op, int out_f16, const void* xq, const void* wq, const float* x_scale,
+                        const float* w_scale, const void* bias, int bias_dtype, void* y, int64_t M, int64_t N,
+                        int64_t K, void* stream) {
+  if (M < 0 || N < 0 || K < 0) return fail("%s: negative dimension", op);
+  if (M > kIntMax || N > kIntMax || K > kIntMax) return fail("%s: dimension exceeds 2^31-1", op);
+  if (bias_dtype < 0 || bias_dtype > 2) return fail("%s: bad bias dtype code %d", op, bias_dtype);
+  if ((bias_dtype != 0) != (bias != nullptr)) return fail("%s: bias pointer and bias dtype disagree", op);
   hipStream_t s = (hipStream_t)stream;
   if (M == 0 || N == 0) return 0;
-  if (!y) return fail("f8f8bf16_rowwise: null output");
+  if (!y) return fail("%s: null output", op);
   if (K == 0) return check_hip(launch_fill_zero_bf16((uint16_t*)y, M * N, s), "zero fill");
-  if (!xq || !wq || !x_scale || !w_scale) return fail("f8f8bf16_rowwise: null pointer");
+  if (!xq || !wq || !x_scale || !w_scale) return fail("%s: null pointer", op);
   GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
-                (int)M, (int)N, (int)K, bias_dtype};
+                (int)M, (int)N, (int)K, bias_dtype, out_f16};
   if (skinny_supports(p)) return check_hip(launch_skinny(p, s), "skinny launch");
   if (dense_tiled_supports(p)) return check_hip(launch_dense_tiled(p, s), "tiled launch");
   return check_hip(launch_generic(p, s), "generic launch");
+}
+
+int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                              void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
+  return rowwise_impl("f8f8bf16_rowwise", 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+}
+
+int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                             const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                             void* stream) {
+  return rowwise_impl("f8f8f16_rowwise", 1, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
 }
 
 int mslk_amd_f8f8bf16_rowwise_grouped(int G, const void* const* xq, const void* const* wq,
@@ -124,7 +136,7 @@ int mslk_amd_f8f8bf16_rowwise_grouped(int G, const void* const* xq, const void* 
     }
     if (!xq[g] || !wq[g] || !x_scale[g] || !w_scale[g]) return fail("f8f8bf16_rowwise_grouped: null pointer in group %d", g);
     GemmProblem p{(const uint8_t*)xq[g], (const uint8_t*)wq[g], x_scale[g], w_scale[g], nullptr, (uint16_t*)y[g],
-                  (int)M[g], (int)N[g], (int)K[g], 0};
+                  (int)M[g], (int)N[g], (int)K[g], 0, 0};
     if (!dense_tiled_supports(p)) {  // odd K or alignment: per-group fallback
       if (int rc = check_hip(launch_generic(p, s), "generic launch")) return rc;
       continue;
@@ -178,6 +190,25 @@ int mslk_amd_f8f8bf16_rowwise_grouped_mm(const void* xq, const void* wq, const f
   DeviceGroups p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, nullptr, (uint16_t*)y, offsets_dev, G,
                  (int)M, (int)N, (int)K, 0, 0};
   return check_hip(launch_device_groups(p, layout, s), "grouped_mm launch");
+}
+
+int mslk_amd_f8f8bf16_rowwise_grouped_dynamic(const void* xq, const void* wq, const float* x_scale,
+                                              const float* w_scale, const int64_t* zero_start_index_M_dev, int G,
+                                              int64_t M, int64_t N, int64_t K, void* y, int zeroing_output,
+                                              void* stream) {
+  if (G < 0 || M < 0 || N < 0 || K < 0) return fail("f8f8bf16_rowwise_grouped_dynamic: negative dimension");
+  if (M > kIntMax || N > kIntMax || K > kIntMax) return fail("f8f8bf16_rowwise_grouped_dynamic: dimension exceeds 2^31-1");
+  hipStream_t s = (hipStream_t)stream;
+  if (G == 0 || M == 0 || N == 0) return 0;
+  if (!y) return fail("f8f8bf16_rowwise_grouped_dynamic: null output");
+  if ((double)G * (double)M * (double)N > 9.0e18) return fail("f8f8bf16_rowwise_grouped_dynamic: output too large");
+  if ((K > 0 && (!xq || !wq)) || !x_scale || !w_scale || !zero_start_index_M_dev)
+    return fail("f8f8bf16_rowwise_grouped_dynamic: null pointer");
+  if (zeroing_output)
+    if (int rc = check_hip(launch_fill_zero_bf16((uint16_t*)y, (int64_t)G * M * N, s), "zero fill")) return rc;
+  DeviceGroups p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, nullptr, (uint16_t*)y, zero_start_index_M_dev,
+                 G, (int)M, (int)N, (int)K, 0, 0};
+  return check_hip(launch_device_groups(p, kGroupsPrepadM, s), "grouped dynamic launch");
 }
 
 int mslk_amd_f8f8bf16_rowwise_batched(const void* xq, const void* wq, const float* x_scale, const float* w_scale,

@@ -45,4 +45,20 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
+// fp32 -> fp16, round to nearest even, overflow to infinity (v_cvt_f16_f32 in the default rounding mode).
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  return (uint32_t)__builtin_bit_cast(unsigned short, (_Float16)f);
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float a, float b) { return f32_to_f16_bits(a) | (f32_to_f16_bits(b) << 16); }
+
+// 16-bit output element of the GEMMs: bf16 (F16 = false) or fp16 (F16 = true).
+template <bool F16>
+__device__ __forceinline__ uint32_t pack_out_x2(float a, float b) {
+  if constexpr (F16) return pack_f16x2(a, b);
+  else return pack_bf16x2(a, b);
+}
+__device__ __forceinline__ uint32_t f32_to_out_bits(float v, int out_f16) {
+  return out_f16 ? f32_to_f16_bits(v) : f32_to_bf16_bits(v);
+}
+
 }  // namespace mslk_amd

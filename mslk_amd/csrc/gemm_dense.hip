@@ -32,6 +32,7 @@ __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p
   if (!map_tile(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
   GemmTile<TS, BIAS> tile;
+  tile.out_f16 = p.out_f16;
   const void* bias = nullptr;
   if constexpr (BIAS == 1) bias = reinterpret_cast<const float*>(p.bias) + n0;
   if constexpr (BIAS == 2) bias = reinterpret_cast<const uint16_t*>(p.bias) + n0;
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(256) void generic_kernel(GemmProblem p) {
   float v = (acc * p.xs[m]) * p.ws[n];
   if (p.bias_dtype == 1) v += reinterpret_cast<const float*>(p.bias)[n];
   else if (p.bias_dtype == 2) v += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]);
-  p.y[idx] = (uint16_t)f32_to_bf16_bits(v);
+  p.y[idx] = (uint16_t)f32_to_out_bits(v, p.out_f16);
 }
 
 __global__ void fill_zero_kernel(uint16_t* y, int64_t n) {

@@ -57,6 +57,7 @@ __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
 //   kGroupsOffsetsN  XQ [G, M, K]; int32 cumulative ends of row blocks of WQ [sum N, K]; Y [M, sum N]
 //   kGroupsOffsetsK  XQ [M, sum K], WQ [N, sum K]; int32 cumulative ends of K slices; Y [G, M, N]
 //   kGroupsUniform   XQ [G, M, K], WQ [G, N, K], Y [G, M, N]
+//   kGroupsPrepadM   as uniform, but only the first layout[g] (int64) rows of group g are computed
 // Scales follow the operand they belong to ([sum M] or [G, M]; [sum N] or [G, N]).
 struct GroupSpan {
   int gi;        // group
@@ -68,7 +69,7 @@ struct GroupSpan {
 template <int LAYOUT, int BM, int BN>
 MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
-  if constexpr (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK) {
+  if constexpr (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK || LAYOUT == kGroupsPrepadM) {
     const int per = tiles_m * tiles_n;
     sp.gi = t / per;
     sp.t = t - sp.gi * per;
@@ -76,6 +77,11 @@ MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
     if constexpr (LAYOUT == kGroupsUniform) {
       sp.o0 = 0;
       sp.len = 0;
+      return true;
+    } else if constexpr (LAYOUT == kGroupsPrepadM) {
+      const int64_t live = static_cast<const int64_t*>(p.layout)[sp.gi];
+      sp.o0 = 0;
+      sp.len = (int)(live < 0 ? 0 : (live > p.M ? p.M : live));
       return true;
     } else {
       const int32_t* off = static_cast<const int32_t*>(p.layout);
@@ -134,7 +140,7 @@ __global__ __launch_bounds__(256) void grouped_device_kernel(DeviceGroups p) {
   using TS = TileShape<BM, BN>;
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
   int t = blockIdx.x;
-  if constexpr (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK) {
+  if constexpr (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK || LAYOUT == kGroupsPrepadM) {
     // The tile count is known on the host: XCD x works on a contiguous slice of the tile list.
     const int total = p.G * ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
     const int per_xcd = (total + kXcds - 1) / kXcds;
@@ -144,12 +150,15 @@ __global__ __launch_bounds__(256) void grouped_device_kernel(DeviceGroups p) {
   GroupSpan sp;
   if (!find_group<LAYOUT, BM, BN>(p, t, sp)) return;
   const int64_t g = sp.gi, M = p.M, N = p.N, K = p.K;
-  const int Mg = (LAYOUT == kGroupsSizesM || LAYOUT == kGroupsOffsetsM) ? sp.len : p.M;
+  const int Mg = (LAYOUT == kGroupsSizesM || LAYOUT == kGroupsOffsetsM || LAYOUT == kGroupsPrepadM) ? sp.len : p.M;
   const int Ng = LAYOUT == kGroupsOffsetsN ? sp.len : p.N;
   const int Kg = LAYOUT == kGroupsOffsetsK ? sp.len : p.K;
   int tm, tn;
-  local_tile(sp.t, (Mg + BM - 1) / BM, (Ng + BN - 1) / BN, tm, tn);
+  local_tile(sp.t, ((LAYOUT == kGroupsPrepadM ? p.M : Mg) + BM - 1) / BM, (Ng + BN - 1) / BN, tm, tn);
   const int64_t m0 = tm * BM, n0 = tn * BN;
+  if constexpr (LAYOUT == kGroupsPrepadM) {
+    if (m0 >= sp.len) return;   // tile of padding rows only
+  }
   const uint8_t *a, *b;
   const float *xs, *ws;
   uint16_t* y;
@@ -188,7 +197,7 @@ template <int LAYOUT, int BM, int BN, int BIAS>
 hipError_t launch_device_shape(const DeviceGroups& p, hipStream_t s) {
   const int64_t tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   int64_t grid;
-  if (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK) {
+  if (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK || LAYOUT == kGroupsPrepadM) {
     grid = (p.G * tiles_m * tiles_n + kXcds - 1) / kXcds * kXcds;
   } else if (LAYOUT == kGroupsOffsetsN) {
     grid = tiles_m * (tiles_n + p.G);   // every group may end in a partial tile
@@ -238,6 +247,7 @@ hipError_t launch_device_groups(const DeviceGroups& in, int layout, hipStream_t 
     case kGroupsOffsetsM: return launch_device_layout<kGroupsOffsetsM, 0>(p, s);
     case kGroupsOffsetsN: return launch_device_layout<kGroupsOffsetsN, 0>(p, s);
     case kGroupsOffsetsK: return launch_device_layout<kGroupsOffsetsK, 0>(p, s);
+    case kGroupsPrepadM: return launch_device_layout<kGroupsPrepadM, 0>(p, s);
     case kGroupsUniform:
       if (p.bias_dtype == 1) return launch_device_layout<kGroupsUniform, 1>(p, s);
       if (p.bias_dtype == 2) return launch_device_layout<kGroupsUniform, 2>(p, s);

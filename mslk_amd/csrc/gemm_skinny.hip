@@ -158,7 +158,7 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
     for (int w = 0; w < kWaves; ++w) sum += red[w][tn][tm][t];
     float val = (sum * e_xs[r]) * e_ws[r];
     if constexpr (BIAS != 0) val += e_b[r];
-    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_bf16_bits(val);
+    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_out_bits(val, p.out_f16);
   }
 }
 
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
     for (int w = 0; w < kWaves; ++w) sum += reinterpret_cast<const float*>(lds + w * XBUF)[frag * 256 + t];
     float val = (sum * e_xs[r]) * e_ws[r];
     if constexpr (BIAS != 0) val += e_b[r];
-    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_bf16_bits(val);
+    p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_out_bits(val, p.out_f16);
   }
 }
 

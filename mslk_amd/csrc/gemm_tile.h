@@ -68,6 +68,7 @@ struct GemmTile {
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
   uint32_t b_off[TS::LB];
+  int out_f16 = 0;          // output element type: 0 bf16, 1 fp16 (set by the caller before run())
   const uint8_t* a_base;    // XQ + m0 * K   (wave-uniform)
   const uint8_t* b_base;    // WQ + n0 * K
 
@@ -283,12 +284,17 @@ struct GemmTile {
     const bool vec16 = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     const bool full = n_rem >= TS::kBN && vec16 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
                       (BIAS == 0 || (reinterpret_cast<uintptr_t>(bias) & (BIAS == 1 ? 15 : 7)) == 0);
-    if (full) epilogue_impl<true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
-    else epilogue_impl<false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+    if (out_f16) {
+      if (full) epilogue_impl<true, true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else epilogue_impl<false, true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+    } else {
+      if (full) epilogue_impl<true, false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else epilogue_impl<false, false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+    }
   }
 
   // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged.
-  template <bool FULL>
+  template <bool FULL, bool F16>
   MSLK_AMD_DEVINL void epilogue_impl(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                      const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     constexpr int WN = TS::kBN / TS::WN;         // columns per wave
@@ -349,8 +355,8 @@ struct GemmTile {
           if constexpr (BIAS != 0) v[r] += bv[tn][r];
         }
         uint2 pk;
-        pk.x = pack_bf16x2(v[0], v[1]);
-        pk.y = pack_bf16x2(v[2], v[3]);
+        pk.x = pack_out_x2<F16>(v[0], v[1]);
+        pk.y = pack_out_x2<F16>(v[2], v[3]);
         *reinterpret_cast<uint2*>(b + j * PITCH + (tn * 16 + 4 * q) * 2) = pk;
       }
       // the buffer is private to the wave: LDS operations of one wave complete in order

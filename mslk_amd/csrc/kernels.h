@@ -25,6 +25,7 @@ struct GemmProblem {
   uint16_t* y;
   int M, N, K;
   int bias_dtype;     // 0 none, 1 fp32, 2 bf16
+  int out_f16;        // 0: Y is bf16, 1: Y is fp16
 };
 
 // Shape classes; each returns hipErrorInvalidValue when the shape is outside what it supports.
@@ -60,6 +61,7 @@ enum GroupLayout : int {
   kGroupsOffsetsN = 2,
   kGroupsOffsetsK = 3,
   kGroupsUniform = 4,
+  kGroupsPrepadM = 5,
 };
 struct DeviceGroups {
   const uint8_t* xq;
@@ -68,7 +70,7 @@ struct DeviceGroups {
   const float* ws;
   const void* bias;     // [G, N], uniform layout only
   uint16_t* y;
-  const void* layout;   // int64 sizes, int32 cumulative ends, or nullptr
+  const void* layout;   // int64 sizes / live-row counts, int32 cumulative ends, or nullptr
   int G;
   int M, N, K;          // the varying dimension holds the total over all groups
   int bias_dtype;       // 0 none, 1 fp32, 2 bf16

@@ -1,6 +1,6 @@
 """`torch.ops.mslk.*` rowwise FP8 GEMM operators backed by the gfx950 HIP kernels.
 
-The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-42,95-96), so callers written
+The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-44,88-89,95-96), so callers written
 against `torch.ops.mslk.f8f8bf16_rowwise` etc. run unchanged.  When the reference's own library has
 already defined a schema, only the GPU ("CUDA" dispatch key) kernel is replaced -- the same seam
 the reference's Python kernels use (mslk/gemm/flydsl/preshuffle_gemm.py:433-475).
@@ -26,9 +26,11 @@ FP8_DTYPE = torch.float8_e4m3fn
 _SCHEMAS = {
     "f8f8bf16_rowwise": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
     "f8f8bf16_rowwise_out": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor(a!) output, Tensor? bias=None, bool use_fast_accum=True) -> ()",
+    "f8f8f16_rowwise": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
     "f8f8bf16_rowwise_grouped": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor[]",
     "f8f8bf16_rowwise_grouped_cat": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor",
     "f8f8bf16_rowwise_grouped_stacked": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor M_sizes) -> Tensor",
+    "f8f8bf16_rowwise_grouped_dynamic": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor zero_start_index_M, bool zeroing_output_tensor=True) -> Tensor",
     "f8f8bf16_rowwise_grouped_mm": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? offsets, Tensor(a!) output) -> Tensor",
     "f8f8bf16_rowwise_batched": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True, Tensor(a!)? output=None) -> Tensor",
 }
@@ -72,7 +74,7 @@ def _bias_args(bias: Optional[torch.Tensor], N: int, device: torch.device):
     return b.data_ptr(), (1 if b.dtype == torch.float32 else 2), b
 
 
-def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None):
+def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, out_dtype=torch.bfloat16):
     _check(XQ.dtype == WQ.dtype, f"XQ and WQ dtypes must match, got {XQ.dtype} vs {WQ.dtype}")
     _check(XQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ.dtype}")
     _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
@@ -94,24 +96,29 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None):
         # empty problem: zeros of the output shape (fp8fp8bf16_rowwise_gemm.hip:531-534)
         if output is not None:
             return output
-        return torch.zeros(out_sizes, dtype=torch.bfloat16, device=XQ.device)
+        return torch.zeros(out_sizes, dtype=out_dtype, device=XQ.device)
     if output is not None:
         Y = output
         y_m = 1
         for d in Y.shape[:-1]:
             y_m *= d
         _check(y_m == M and Y.shape[-1] == N, "output has the wrong shape")
-        _check(Y.dtype == torch.bfloat16, "output must be bfloat16")
+        _check(Y.dtype == out_dtype, f"output must be {out_dtype}")
         _check(Y.is_cuda and Y.is_contiguous() and Y.device == XQ.device, "output must be a contiguous GPU tensor")
     else:
-        Y = torch.empty(out_sizes, dtype=torch.bfloat16, device=XQ.device)
+        Y = torch.empty(out_sizes, dtype=out_dtype, device=XQ.device)
     xs = x_scale.contiguous()
     ws = w_scale.contiguous()
     bias_ptr, bias_code, _keep = _bias_args(bias, N, XQ.device)
     with _on_device(XQ.device):
-        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise(
-            XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
-            M, N, K, None, 0, _stream_ptr(XQ.device)))
+        if out_dtype == torch.float16:
+            _lib.check(_lib.lib().mslk_amd_f8f8f16_rowwise(
+                XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
+                M, N, K, _stream_ptr(XQ.device)))
+        else:
+            _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise(
+                XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
+                M, N, K, None, 0, _stream_ptr(XQ.device)))
     return Y
 
 
@@ -121,6 +128,11 @@ def f8f8bf16_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
 
 def f8f8bf16_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_accum=True):
     _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output)
+
+
+def f8f8f16_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
+    """Same GEMM with an fp16 result (fp8fp8fp16_rowwise_gemm.hip:66-133)."""
+    return _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, None, torch.float16)
 
 
 def _check_grouped(XQ: Sequence[torch.Tensor], WQ, x_scale, w_scale):
@@ -291,6 +303,36 @@ def f8f8bf16_rowwise_grouped_mm(XQ, WQ, x_scale, w_scale, offsets, output) -> to
     return output
 
 
+def f8f8bf16_rowwise_grouped_dynamic(XQ, WQ, x_scale, w_scale, zero_start_index_M, zeroing_output_tensor=True) -> torch.Tensor:
+    """XQ [G, M, K], WQ [G, N, K] -> bf16 [G, M, N]; only the first zero_start_index_M[g] rows of group
+    g are computed, the others are zero (or uninitialised when zeroing_output_tensor is False).
+    Deprecated in the reference (fp8_rowwise_grouped_gemm.hip:656-714) but still registered."""
+    _check(XQ.dim() == 3, "Input XQ must be 3D (G,M,K).")
+    _check(WQ.dim() == 3, "Input WQ must be 3D (G,N,K).")
+    _check(XQ.is_cuda and XQ.is_contiguous() and WQ.is_cuda and WQ.is_contiguous(), "XQ/WQ must be contiguous GPU tensors")
+    _check(XQ.dtype == WQ.dtype, f"XQ and WQ dtypes must match, got {XQ.dtype} vs {WQ.dtype}")
+    _check(XQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ.dtype}")
+    _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
+    G, M, K = XQ.shape
+    N = WQ.shape[1]
+    _check(WQ.shape[0] == G and x_scale.numel() == G * M and w_scale.numel() == G * N and WQ.shape[2] == K,
+           "All inputs must have the same number of groups.")
+    _check(N >= 512 and K >= 512, "N and K must be at least 512 for grouped gemm. For smaller inputs, consider unrolling.")
+    zs = zero_start_index_M
+    _check(zs.is_cuda and zs.dtype == torch.int64 and zs.numel() == G, "zero_start_index_M must be an int64 GPU tensor with G entries")
+    _check(WQ.device == XQ.device and x_scale.device == XQ.device and w_scale.device == XQ.device and zs.device == XQ.device,
+           "all operands must be on the same device")
+    Y = torch.empty((G, M, N), dtype=torch.bfloat16, device=XQ.device)
+    if Y.numel() == 0:
+        return Y
+    xs, ws, zs = x_scale.contiguous(), w_scale.contiguous(), zs.contiguous()
+    with _on_device(XQ.device):
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped_dynamic(
+            XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), zs.data_ptr(), G, M, N, K, Y.data_ptr(),
+            1 if zeroing_output_tensor else 0, _stream_ptr(XQ.device)))
+    return Y
+
+
 def f8f8bf16_rowwise_batched(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True, output=None) -> torch.Tensor:
     """XQ [B, M, K], WQ [B, N, K], x_scale [B, M], w_scale [B, N] -> bf16 [B, M, N]
     (fp8_rowwise_batched_gemm.hip:199-254).  `bias` [B, N] (fp32 or bf16) is added per batch as the
@@ -334,9 +376,11 @@ def f8f8bf16_rowwise_batched(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum
 _IMPLS = {
     "f8f8bf16_rowwise": f8f8bf16_rowwise,
     "f8f8bf16_rowwise_out": f8f8bf16_rowwise_out,
+    "f8f8f16_rowwise": f8f8f16_rowwise,
     "f8f8bf16_rowwise_grouped": f8f8bf16_rowwise_grouped,
     "f8f8bf16_rowwise_grouped_cat": f8f8bf16_rowwise_grouped_cat,
     "f8f8bf16_rowwise_grouped_stacked": f8f8bf16_rowwise_grouped_stacked,
+    "f8f8bf16_rowwise_grouped_dynamic": f8f8bf16_rowwise_grouped_dynamic,
     "f8f8bf16_rowwise_grouped_mm": f8f8bf16_rowwise_grouped_mm,
     "f8f8bf16_rowwise_batched": f8f8bf16_rowwise_batched,
 }
@@ -345,6 +389,11 @@ _IMPLS = {
 def _fake_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
     # mslk/gemm/_meta.py:26-50, generalised to any number of leading dims
     return torch.empty(tuple(XQ.shape[:-1]) + (WQ.shape[0],), dtype=torch.bfloat16, device=XQ.device)
+
+
+def _fake_rowwise_f16(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
+    # mslk/gemm/_meta.py:516-529, generalised to any number of leading dims
+    return torch.empty(tuple(XQ.shape[:-1]) + (WQ.shape[0],), dtype=torch.float16, device=XQ.device)
 
 
 def _fake_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_accum=True):
@@ -364,6 +413,10 @@ def _fake_grouped_stacked(XQ, WQ, x_scale, w_scale, M_sizes):
     return torch.empty((XQ.shape[0], WQ.shape[1]), dtype=torch.bfloat16, device=XQ.device)
 
 
+def _fake_grouped_dynamic(XQ, WQ, x_scale, w_scale, zero_start_index_M, zeroing_output_tensor=True):
+    return torch.empty((XQ.shape[0], XQ.shape[1], WQ.shape[1]), dtype=torch.bfloat16, device=XQ.device)
+
+
 def _fake_grouped_mm(XQ, WQ, x_scale, w_scale, offsets, output):
     return output
 
@@ -378,9 +431,11 @@ def _fake_batched(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True, outp
 _FAKES = {
     "f8f8bf16_rowwise": _fake_rowwise,
     "f8f8bf16_rowwise_out": _fake_rowwise_out,
+    "f8f8f16_rowwise": _fake_rowwise_f16,
     "f8f8bf16_rowwise_grouped": _fake_grouped,
     "f8f8bf16_rowwise_grouped_cat": _fake_grouped_cat,
     "f8f8bf16_rowwise_grouped_stacked": _fake_grouped_stacked,
+    "f8f8bf16_rowwise_grouped_dynamic": _fake_grouped_dynamic,
     "f8f8bf16_rowwise_grouped_mm": _fake_grouped_mm,
     "f8f8bf16_rowwise_batched": _fake_batched,
 }

@@ -68,7 +68,12 @@ def test_ops_registered_with_reference_schemas():
     s = str(torch.ops.mslk.f8f8bf16_rowwise_batched.default._schema)
     assert s == ("mslk::f8f8bf16_rowwise_batched(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
                  "Tensor? bias=None, bool use_fast_accum=True, Tensor(a!)? output=None) -> Tensor")
-    assert hasattr(torch.ops.mslk, "quantize_fp8_row")
+    s = str(torch.ops.mslk.f8f8f16_rowwise.default._schema)
+    assert s == ("mslk::f8f8f16_rowwise(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
+                 "Tensor? bias=None, bool use_fast_accum=True) -> Tensor")
+    s = str(torch.ops.mslk.f8f8bf16_rowwise_grouped_dynamic.default._schema)
+    assert s.endswith("Tensor zero_start_index_M, bool zeroing_output_tensor=True) -> Tensor")
+    assert hasattr(torch.ops.mslk, "quantize_fp8_row") and hasattr(torch.ops.mslk, "dequantize_fp8_row")
 
 
 def test_fake_kernels_give_reference_shapes():

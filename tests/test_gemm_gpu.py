@@ -245,3 +245,45 @@ def test_cfg3_decode(M):
     y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
     torch.cuda.synchronize()
     assert_gemm_close(y, O.dequant_matmul(rq, wq.cpu(), rs, ws.cpu()), f"cfg3 M={M}")
+
+
+@pytest.mark.parametrize("M,N,K", [(512, 512, 256), (300, 260, 384), (16, 512, 512), (40, 300, 1040), (33, 20, 50),
+                                   (1, 8192, 1024), (2048, 1024, 512)])
+def test_fp16_output_exact_cases_and_overflow(M, N, K):
+    """f8f8f16_rowwise on inputs whose fp32 result is exact: the output must be the fp16 rounding
+    (nearest even, overflow to infinity) of that result, bit for bit.  The scales reach 2^6, so some
+    outputs exceed 65504 and must come out infinite."""
+    g = torch.Generator().manual_seed(K + 1)
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    xs = 2.0 ** torch.randint(-9, 7, (M,), generator=g).float()
+    ws = 2.0 ** torch.randint(-9, 7, (N,), generator=g).float()
+    bias = torch.randint(-4, 5, (N,), generator=g).float() * 2.0 ** -5
+    want = ((xi @ wi.T) * xs[:, None] * ws[None, :] + bias[None, :]).to(torch.float16)
+    y = torch.ops.mslk.f8f8f16_rowwise(*_gpu(xi.to(F8), wi.to(F8), xs, ws), bias=bias.to(DEV))
+    torch.cuda.synchronize()
+    assert y.dtype == torch.float16 and y.shape == (M, N)
+    assert torch.equal(y.cpu().view(torch.int16), want.view(torch.int16))
+    if M * N >= 512 * 512:
+        assert torch.isinf(want).any() and (want.abs() < 2.0 ** -14).any()   # overflow and subnormal results both occur
+
+
+@pytest.mark.parametrize("M,N,K", [(4096, 4096, 4096), (300, 517, 256), (64, 8192, 8192), (5, 8200, 5120), (65, 33, 17)])
+def test_fp16_output_matches_oracle(M, N, K):
+    g = torch.Generator().manual_seed(M + N + K)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    y = torch.ops.mslk.f8f8f16_rowwise(*_gpu(xq, wq, xs, ws))
+    yb = torch.ops.mslk.f8f8bf16_rowwise(*_gpu(xq, wq, xs, ws))
+    torch.cuda.synchronize()
+    ref = O.dequant_matmul(xq, wq, xs, ws)
+    assert_gemm_close(y, ref, "fp16 out")
+    _, normwise = O.gemm_errors(y.float().cpu(), ref)
+    assert normwise <= 5e-4   # fp16 keeps 10 mantissa bits: only the accumulation error is left
+    # both outputs are roundings of the same fp32 value v: |fp16(v) - v| <= 2^-11 |v| and |bf16(v) - v| <= 2^-8 |v|,
+    # and re-rounding the fp16 result to bf16 lands on another bf16 than the direct rounding only when
+    # v lies within half an fp16 ulp of a bf16 rounding boundary (1 value in 16 for a smooth distribution)
+    yf, ybf = y.float(), yb.float()
+    normal = yf.abs() >= 2.0 ** -14
+    assert ((yf - ybf).abs()[normal] <= yf.abs()[normal] * (2.0 ** -8 + 2.0 ** -11) * 1.0001).all()
+    differs = (yf.bfloat16() != yb).float().mean().item()
+    assert differs < 0.09

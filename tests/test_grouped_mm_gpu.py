@@ -138,6 +138,24 @@ def test_2d_2d_offsets_over_k(ks, M, N):
             assert (y[gi] == 0).all()   # empty sum
 
 
+@pytest.mark.parametrize("G,M,N,K,live", [(4, 300, 512, 512, [300, 0, 17, 256]), (2, 64, 768, 1024, [1, 64]),
+                                          (3, 700, 520, 656, [513, 700, 255])])
+def test_grouped_dynamic_prepadded_rows(G, M, N, K, live):
+    g = torch.Generator().manual_seed(G + M + N + K)
+    xq, xs = _quant(G * M, K, g)
+    wq, ws = _quant(G * N, K, g, 0.02)
+    zs = torch.tensor(live, dtype=torch.int64, device=DEV)
+    y = torch.ops.mslk.f8f8bf16_rowwise_grouped_dynamic(xq.view(G, M, K).to(DEV), wq.view(G, N, K).to(DEV),
+                                                        xs.view(G, M).to(DEV), ws.view(G, N).to(DEV), zs)
+    torch.cuda.synchronize()
+    assert y.shape == (G, M, N) and y.dtype == torch.bfloat16
+    for gi, m in enumerate(live):
+        if m:
+            rows, cols = slice(gi * M, gi * M + m), slice(gi * N, (gi + 1) * N)
+            assert_gemm_close(y[gi, :m], O.dequant_matmul(xq[rows], wq[cols], xs[rows], ws[cols]), f"group {gi}")
+        assert (y[gi, m:] == 0).all()
+
+
 def test_inconsistent_offsets_write_nothing_out_of_range():
     g = torch.Generator().manual_seed(5)
     M, N, K = 128, 512, 512
