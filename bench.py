@@ -261,6 +261,44 @@ def main():
         extras["dequantize_cfg1"] = {"ms": d_ms, "GBps": q_bytes / (d_ms * 1e-3) / 1e9,
                                      "frac_hbm": q_bytes / (d_ms * 1e-3) / PEAK_HBM_BPS, "bytes": q_bytes}
         del qsets, dq_out
+
+        # fused producers of the MoE activations on cfg4's token count (8192 x 5120, bf16)
+        from mslk_amd import moe
+        Tm, Dm, Em = 8192, 5120, 16
+        gen = torch.Generator(device="cpu").manual_seed(5)
+        h = torch.randn(Tm, 2 * Dm, generator=gen).bfloat16().to(dev)
+        hsets = [h.clone() for _ in range(3)]                       # 3 x 160 MiB
+        fq = torch.empty(Tm, Dm, dtype=torch.float8_e4m3fn, device=dev)
+        fs = torch.empty(Tm, dtype=torch.float32, device=dev)
+
+        def silu_step(i):
+            hh = hsets[i % 3]
+            api.check(api.L.mslk_amd_silu_mul_quant(hh.data_ptr(), hh.data_ptr() + 2 * Dm, 0, Tm, Dm, 2 * Dm, 2 * Dm,
+                                                    fq.data_ptr(), fs.data_ptr(), None, None, 0, api.stream))
+
+        for i in range(6):
+            silu_step(i)
+        f_ms = _median_events_ms(silu_step, 30)
+        f_bytes = 5.0 * Tm * Dm + 4.0 * Tm
+        extras["silu_mul_quant_8192x5120"] = {"ms": f_ms, "GBps": f_bytes / (f_ms * 1e-3) / 1e9,
+                                              "frac_hbm": f_bytes / (f_ms * 1e-3) / PEAK_HBM_BPS, "bytes": f_bytes}
+        tok = torch.randperm(Tm, generator=gen).to(torch.int32).to(dev)
+        exp = torch.randint(0, Em, (Tm,), generator=gen).to(dev)
+        scores = torch.rand(Tm, Em, generator=gen).to(dev)
+        xsrc = [hsets[j][:, :Dm].contiguous() for j in range(3)]
+
+        def gather_step(i):
+            api.check(api.L.mslk_amd_gather_scale_quant_dense_tokens(
+                xsrc[i % 3].data_ptr(), 0, Tm, Dm, tok.data_ptr(), 1, exp.data_ptr(), 0, Tm, scores.data_ptr(), 2, Em, Em, 1,
+                fq.data_ptr(), fs.data_ptr(), None, None, 0, api.stream))
+
+        for i in range(6):
+            gather_step(i)
+        g_ms = _median_events_ms(gather_step, 30)
+        g_bytes = 3.0 * Tm * Dm + 16.0 * Tm
+        extras["gather_scale_quant_8192x5120"] = {"ms": g_ms, "GBps": g_bytes / (g_ms * 1e-3) / 1e9,
+                                                  "frac_hbm": g_bytes / (g_ms * 1e-3) / PEAK_HBM_BPS, "bytes": g_bytes}
+        del hsets, xsrc, h
         if args.only == "quantize":
             print(json.dumps(extras))
             return

@@ -76,6 +76,40 @@ int mslk_amd_quantize_fp8_row_jagged(const void* x, int x_dtype, int64_t rows, i
 int mslk_amd_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out, void* stream);
 
 /*
+ * Fused SiLU-gate, multiply and row-wise FP8 quantization: the producer of the second MoE GEMM's
+ * activations.  Replaces mslk::silu_mul_quant (reference: mslk/moe/activation.py:72-135 wrapper,
+ * 232-300 kernel):
+ *   y = x0 * sigmoid(x0) * x1 in fp32;  row_max = clamp(max|y|, 1e-12 [, *scale_ub]);  s = 448 / row_max;
+ *   out = e4m3fn_rne(clamp(y * s, -448, 448));  out_scale = 1 / s.
+ *   x0, x1     [T, D] bf16 or fp16 (x_dtype), unit column stride, row strides in elements
+ *   out        [T, D] e4m3fn contiguous;  out_scale [T] fp32
+ *   valid_token_count  optional device scalar (int32 or int64 per count_dtype): rows at or beyond it
+ *                      are neither read nor written
+ */
+int mslk_amd_silu_mul_quant(const void* x0, const void* x1, int x_dtype, int64_t T, int64_t D, int64_t x0_row_stride,
+                            int64_t x1_row_stride, void* out, float* out_scale, const float* scale_ub,
+                            const void* valid_token_count, int count_dtype, void* stream);
+
+/*
+ * Fused gather of routed tokens, multiplication by the routing score and row-wise FP8 quantization:
+ * the producer of the first MoE GEMM's activations.  Replaces gather_scale_quant_dense_tokens
+ * (reference: mslk/moe/gather_scatter.py:96-170 wrapper, 545-640 kernel):
+ *   y[i] = x[token_indices[i]] * scores[token_indices[i], expert_indices[i]] in fp32, then quantized
+ *   as in mslk_amd_silu_mul_quant.
+ *   x [T, D] bf16/fp16 contiguous; token_indices, expert_indices [a] int32 or int64 (per *_dtype);
+ *   scores [T, E] bf16/fp16/fp32 with element strides (score_stride_t, score_stride_e);
+ *   out [a, D] e4m3fn; out_scale [a].  Rows at or beyond *valid_token_count, and rows whose indices fall
+ *   outside [0, T) x [0, E), are neither read nor written.
+ */
+int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t T, int64_t D,
+                                             const void* token_indices, int token_dtype,
+                                             const void* expert_indices, int expert_dtype, int64_t a,
+                                             const void* scores, int score_dtype, int64_t E, int64_t score_stride_t,
+                                             int64_t score_stride_e, void* out, float* out_scale,
+                                             const float* scale_ub, const void* valid_token_count, int count_dtype,
+                                             void* stream);
+
+/*
  * Dense rowwise-scaled FP8 GEMM.  Replaces mslk::gemm::f8f8bf16_rowwise / f8f8bf16_rowwise_out
  * (reference: csrc/gemm/gemm_ops.cpp:31-34; host wrapper csrc/gemm/ck/fp8_rowwise/fp8fp8bf16_rowwise_gemm.hip:499-576;
  * math csrc/gemm/ck/fp8_rowwise/kernels/fp8_rowwise_common.h:54-82,168-204; bias semantics

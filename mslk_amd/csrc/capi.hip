@@ -77,6 +77,51 @@ int mslk_amd_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows
   return check_hip(launch_dequantize_fp8_row(xq, scale, rows, K, out, (hipStream_t)stream), "dequantize_fp8_row launch");
 }
 
+int mslk_amd_silu_mul_quant(const void* x0, const void* x1, int x_dtype, int64_t T, int64_t D, int64_t x0_row_stride,
+                            int64_t x1_row_stride, void* out, float* out_scale, const float* scale_ub,
+                            const void* valid_token_count, int count_dtype, void* stream) {
+  if (x_dtype != MSLK_AMD_DTYPE_BF16 && x_dtype != MSLK_AMD_DTYPE_F16)
+    return fail("silu_mul_quant: inputs must be bf16 or fp16 (dtype code %d)", x_dtype);
+  if (count_dtype != MSLK_AMD_INDEX_I64 && count_dtype != MSLK_AMD_INDEX_I32)
+    return fail("silu_mul_quant: unsupported valid_token_count dtype code %d", count_dtype);
+  if (T < 0 || D < 0) return fail("silu_mul_quant: negative dimension");
+  if (T > kIntMax || D > kIntMax) return fail("silu_mul_quant: dimension exceeds 2^31-1");
+  if (T == 0 || D == 0) return 0;
+  if (!x0 || !x1 || !out || !out_scale) return fail("silu_mul_quant: null pointer");
+  if (x0_row_stride < D || x1_row_stride < D) return fail("silu_mul_quant: row stride smaller than D");
+  FusedQuantArgs p{};
+  p.x0 = x0; p.x1 = x1; p.stride0 = x0_row_stride; p.stride1 = x1_row_stride; p.dtype = x_dtype;
+  p.out = (uint8_t*)out; p.out_scale = out_scale; p.rows = T; p.D = (int)D; p.scale_ub = scale_ub;
+  p.valid_count = valid_token_count; p.valid_is_i64 = count_dtype == MSLK_AMD_INDEX_I64;
+  return check_hip(launch_fused_quant(p, kFusedSiluMul, (hipStream_t)stream), "silu_mul_quant launch");
+}
+
+int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t T, int64_t D,
+                                             const void* token_indices, int token_dtype,
+                                             const void* expert_indices, int expert_dtype, int64_t a,
+                                             const void* scores, int score_dtype, int64_t E, int64_t score_stride_t,
+                                             int64_t score_stride_e, void* out, float* out_scale,
+                                             const float* scale_ub, const void* valid_token_count, int count_dtype,
+                                             void* stream) {
+  const char* op = "gather_scale_quant_dense_tokens";
+  if (x_dtype != MSLK_AMD_DTYPE_BF16 && x_dtype != MSLK_AMD_DTYPE_F16) return fail("%s: x must be bf16 or fp16 (dtype code %d)", op, x_dtype);
+  if (score_dtype < 0 || score_dtype > 2) return fail("%s: unsupported scores dtype code %d", op, score_dtype);
+  if ((token_dtype | expert_dtype | count_dtype) & ~1) return fail("%s: index dtype codes must be MSLK_AMD_INDEX_I64 or _I32", op);
+  if (T < 0 || D < 0 || a < 0 || E < 0) return fail("%s: negative dimension", op);
+  if (a > kIntMax || D > kIntMax) return fail("%s: dimension exceeds 2^31-1", op);
+  if (a == 0 || D == 0) return 0;
+  if (!x || !token_indices || !expert_indices || !scores || !out || !out_scale) return fail("%s: null pointer", op);
+  FusedQuantArgs p{};
+  p.x0 = x; p.stride0 = D; p.dtype = x_dtype;
+  p.out = (uint8_t*)out; p.out_scale = out_scale; p.rows = a; p.D = (int)D; p.scale_ub = scale_ub;
+  p.valid_count = valid_token_count; p.valid_is_i64 = count_dtype == MSLK_AMD_INDEX_I64;
+  p.token_idx = token_indices; p.token_is_i64 = token_dtype == MSLK_AMD_INDEX_I64;
+  p.expert_idx = expert_indices; p.expert_is_i64 = expert_dtype == MSLK_AMD_INDEX_I64;
+  p.scores = scores; p.score_dtype = score_dtype; p.stride_t = score_stride_t; p.stride_e = score_stride_e;
+  p.T = T; p.E = E;
+  return check_hip(launch_fused_quant(p, kFusedGatherScale, (hipStream_t)stream), "gather_scale_quant launch");
+}
+
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
 
 static int rowwise_impl(const char* op, int out_f16, const void* xq, const void* wq, const float* x_scale,

@@ -15,6 +15,32 @@ hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t
                                      hipStream_t s);
 hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t s);
 
+// Fused producers of quantized activations (fused_quant.hip).
+enum FusedQuantOp : int { kFusedSiluMul = 0, kFusedGatherScale = 1 };
+struct FusedQuantArgs {
+  const void* x0;            // silu: gate input [rows, D]; gather: token matrix x [T, D]
+  const void* x1;            // silu: up input [rows, D]
+  int64_t stride0, stride1;  // row strides in elements
+  int dtype;                 // element type of x0 / x1: 0 bf16, 1 fp16
+  uint8_t* out;              // [rows, D] e4m3fn, contiguous
+  float* out_scale;          // [rows]
+  int64_t rows;
+  int D;
+  const float* scale_ub;     // optional
+  const void* valid_count;   // optional device scalar: rows at or beyond it are left untouched
+  int valid_is_i64;
+  // gather only
+  const void* token_idx;     // [rows]
+  int token_is_i64;
+  const void* expert_idx;    // [rows]
+  int expert_is_i64;
+  const void* scores;        // [T, E] with strides (stride_t, stride_e) in elements
+  int score_dtype;           // 0 bf16, 1 fp16, 2 fp32
+  int64_t stride_t, stride_e;
+  int64_t T, E;
+};
+hipError_t launch_fused_quant(const FusedQuantArgs& p, int op, hipStream_t s);
+
 // One GEMM problem: Y[M,N] = bf16(XQ[M,K] . WQ[N,K]^T * xs[:,None] * ws[None,:] + bias[None,:]).
 struct GemmProblem {
   const uint8_t* xq;

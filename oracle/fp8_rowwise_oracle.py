@@ -11,6 +11,10 @@ Every function restates, in plain CPU torch, the arithmetic of one reference fun
   dequant_matmul          test/gemm/triton/fp8_gemm_test.py:126-132     (tight GEMM oracle)
   matmul_fp8_row_cpu      mslk/gemm/triton/fp8_gemm.py:1186-1201        (CPU fallback = timed CPU baseline)
   grouped_*               test/gemm/triton/grouped_gemm_test.py:116-121, bench/gemm/gemm_ops.py:632-644
+  quantize_fp8_row_jagged mslk/quantize/triton/fp8_quantize.py:123-129,236-243
+  dequantize_fp8_row[_bf16] mslk/quantize/triton/fp8_quantize.py:1060-1113
+  quantize_rows_saturating, silu_mul_quant, gather_scale_quant_dense_tokens
+                          mslk/moe/activation.py:232-300, mslk/moe/gather_scatter.py:545-640
 
 Pinning (what keeps this file honest; see tests/test_oracle.py):
   * quantize: the scalar C twin in oracle/fp8_rowwise_oracle.c shares no code with torch and is
@@ -18,6 +22,10 @@ Pinning (what keeps this file honest; see tests/test_oracle.py):
     forms (amax = 448*2^k, zero rows, one-hot rows, -0.0, NaN rows) are asserted separately.
   * dequant_matmul: brute-force float64 triple loop (C twin), identity / one-hot weights,
     integer-valued codes where fp32 accumulation is exact.
+  * jagged / dequantize / saturating quantization: closed forms and hand-worked roundings.
+  * silu_mul_quant: the sigmoid is torch's CPU sigmoid; the reference's Triton sigmoid may differ in
+    the last bits, so parity is unpinned at bit level and held to the reference test's own
+    tolerance (test/moe/activation_test.py:168-170) plus a bound on the fraction of differing codes.
   * matmul_fp8_row_cpu: parity unpinned at bit level (it is a timing baseline whose bf16 matmul
     rounds before scaling); it is only checked to agree with dequant_matmul within bf16 tolerance.
 """
@@ -78,6 +86,44 @@ def quantize_fp8_row_jagged(a: torch.Tensor, zero_start_index_M: torch.Tensor,
     live = n < zs[:, :, None]
     masked = torch.where(live[..., None], a4, torch.zeros((), dtype=a.dtype)).reshape(a.shape)
     return quantize_fp8_row(masked, scale_ub)
+
+
+def quantize_rows_saturating(y: torch.Tensor, scale_ub: Optional[torch.Tensor] = None
+                             ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Row-wise quantization as written inside the reference's fused MoE kernels
+    (mslk/moe/activation.py:281-297, mslk/moe/gather_scatter.py:601-633), all in fp32:
+        row_max = clamp(max|y|, 1e-12 [, scale_ub]);  s = 448 / row_max;  scale = 1 / s;
+        code = e4m3fn_rne(clamp(y * s, -448, 448)).
+    It differs from quantize_fp8_row (the torch branch) in the order of the two divisions and in that
+    it saturates instead of producing NaN when scale_ub cuts the maximum."""
+    y = y.to(torch.float32)
+    row_max = y.abs().amax(dim=-1)
+    if scale_ub is not None:
+        row_max = torch.clamp(row_max, min=1e-12, max=float(scale_ub.reshape(-1)[0].to(torch.float32)))
+    else:
+        row_max = torch.clamp(row_max, min=1e-12)
+    s = torch.tensor(FP8_MAX, dtype=torch.float32) / row_max
+    q = torch.clamp(y * s[..., None], -FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q, 1.0 / s
+
+
+def silu_mul_quant(x0: torch.Tensor, x1: torch.Tensor, scale_ub: Optional[torch.Tensor] = None
+                   ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """quantize(x0 * sigmoid(x0) * x1), the product taken in fp32 left to right
+    (mslk/moe/activation.py:270-279; the same expression is the reference test's own oracle,
+    test/moe/activation_test.py:159-163)."""
+    a, b = x0.to(torch.float32), x1.to(torch.float32)
+    return quantize_rows_saturating(a * torch.sigmoid(a) * b, scale_ub)
+
+
+def gather_scale_quant_dense_tokens(x: torch.Tensor, token_indices: torch.Tensor, expert_indices: torch.Tensor,
+                                    scores: torch.Tensor, scale_ub: Optional[torch.Tensor] = None
+                                    ) -> Tuple[torch.Tensor, torch.Tensor]:
+    """quantize(x[token] * scores[token, expert]) in fp32 (mslk/moe/gather_scatter.py:564-633; the
+    reference test builds the same product, test/moe/gather_scatter_test.py:170-182)."""
+    t, e = token_indices.to(torch.int64), expert_indices.to(torch.int64)
+    y = x[t].to(torch.float32) * scores[t, e].to(torch.float32)[:, None]
+    return quantize_rows_saturating(y, scale_ub)
 
 
 def dequant_matmul(xq: torch.Tensor, wq: torch.Tensor, x_scale: torch.Tensor,

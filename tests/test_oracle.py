@@ -257,3 +257,58 @@ def test_dequantize_closed_forms():
     back = O.dequantize_fp8_row_bf16(q, sc).float()
     amax = a.float().abs().amax(dim=1, keepdim=True)
     assert ((back - a.float()).abs() <= a.float().abs() * 2.0 ** -4 + amax * 2.0 ** -9).all()
+
+
+def test_saturating_quantization_closed_forms():
+    # amax = 448 * 2^k: s = 2^-k exactly, scale = 2^k, every value v * 2^-k is converted exactly as is
+    for k in (-3, 0, 5):
+        y = torch.tensor([[448.0, -224.0, 1.0, 0.0, 17.0, -0.4375]]) * 2.0 ** k
+        q, sc = O.quantize_rows_saturating(y)
+        assert sc.item() == 2.0 ** k
+        assert q.view(torch.uint8).tolist() == [[0x7E, 0xF6, 0x38, 0x00, 0x58, 0xAE]]   # 17 -> 16 (tie to even), -0.4375 exact
+    # scale_ub below the maximum: larger values saturate at +-448 (0x7E / 0xFE) instead of becoming NaN
+    y = torch.tensor([[100.0, -50.0, 25.0, 10.0]])
+    q, sc = O.quantize_rows_saturating(y, torch.tensor([25.0]))
+    assert sc.item() == torch.tensor(1.0) / (torch.tensor(448.0) / torch.tensor(25.0))
+    assert q.view(torch.uint8)[0, :3].tolist() == [0x7E, 0xFE, 0x7E]
+    assert q.float()[0, 3].item() == 176.0    # 10 * 17.92 = 179.2 -> grid {160, 176, 192}
+    # zero row: the clamp at 1e-12 decides the scale
+    q, sc = O.quantize_rows_saturating(torch.zeros(1, 8))
+    assert (q.view(torch.uint8) == 0).all() and sc.item() == (torch.tensor(1.0) / (torch.tensor(448.0) / torch.tensor(1e-12))).item()
+    # on rows where both formulas are exact they agree with the stand-alone quantizer
+    g = torch.Generator().manual_seed(8)
+    y = torch.randn(16, 64, generator=g)
+    y[:, 0] = 448.0 * 2.0 ** torch.randint(-4, 4, (16,), generator=g).float()
+    y = torch.minimum(y.abs(), y[:, :1]) * torch.sign(y)
+    q1, s1 = O.quantize_rows_saturating(y)
+    q2, s2 = O.quantize_fp8_row(y)
+    assert torch.equal(q1.view(torch.uint8), q2.view(torch.uint8)) and torch.equal(s1, s2)
+
+
+def test_fused_producers_reduce_to_their_parts():
+    g = torch.Generator().manual_seed(9)
+    x0 = torch.randn(5, 40, generator=g).bfloat16()
+    x1 = torch.randn(5, 40, generator=g).bfloat16()
+    q, sc = O.silu_mul_quant(x0, x1)
+    # silu(0) = 0 and silu(x) -> x for large x: closed-form rows
+    big = torch.full((1, 8), 30.0).bfloat16()
+    q2, s2 = O.silu_mul_quant(big, torch.tensor([[1.0, 2.0, 4.0, -8.0, 0.5, 0.0, 1.0, 1.0]]).bfloat16())
+    assert s2.item() == (torch.tensor(1.0) / (torch.tensor(448.0) / torch.tensor(240.0))).item()
+    assert q2.float()[0].tolist() == [56.0, 112.0, 224.0, -448.0, 28.0, 0.0, 56.0, 56.0]
+    qz, _ = O.silu_mul_quant(torch.zeros(1, 8).bfloat16(), big)
+    assert (qz.view(torch.uint8) == 0).all()
+    # independent evaluation in float64
+    y64 = (x0.double() * torch.sigmoid(x0.double()) * x1.double())
+    back = q.float() * sc[:, None]
+    assert ((back - y64.float()).abs() <= y64.abs().float() * 2.0 ** -4 + y64.abs().amax(dim=1, keepdim=True).float() * 2.0 ** -9).all()
+    # gather: a permutation with unit scores is a row permutation of the plain quantization
+    x = torch.randn(7, 32, generator=g).bfloat16()
+    perm = torch.randperm(7, generator=g)
+    qg, sg = O.gather_scale_quant_dense_tokens(x, perm, torch.zeros(7, dtype=torch.int64), torch.ones(7, 1))
+    qp, sp = O.quantize_rows_saturating(x.float())
+    assert torch.equal(qg.view(torch.uint8), qp.view(torch.uint8)[perm]) and torch.equal(sg, sp[perm])
+    # a power-of-two score only moves the scale
+    sc2 = torch.full((7, 3), 1.0)
+    sc2[:, 2] = 4.0
+    qg2, sg2 = O.gather_scale_quant_dense_tokens(x, perm, torch.full((7,), 2), sc2)
+    assert torch.equal(qg2.view(torch.uint8), qg.view(torch.uint8)) and torch.equal(sg2, sg * 4.0)
