@@ -11,7 +11,8 @@
 //   row_max = clamp(max|y|, 1e-12 [, *scale_ub]);  s = 448 / row_max;  out_scale = 1 / s;
 //   code = e4m3fn_rne(clamp(y * s, -448, 448))
 // (saturating, unlike the stand-alone quantizer whose contract is the reference's torch branch).
-// Divisions are IEEE-correct; sigmoid is 1 / (1 + expf(-x)).
+// The two divisions of the scale are IEEE-correct; sigmoid is rcp(1 + exp(-x)) on the hardware
+// transcendental units, accurate to a few fp32 ulp.
 //
 // HBM-bound (silu: 4 B in + 1 B out per element for 16-bit inputs; gather: 2 B in + 1 B out).  One
 // workgroup of 256 lanes owns a row; the produced fp32 values stay in registers between the
@@ -41,8 +42,22 @@ MSLK_AMD_DEVINL int64_t load_index(const void* p, int64_t i, int is_i64) {
   return is_i64 ? static_cast<const int64_t*>(p)[i] : (int64_t) static_cast<const int32_t*>(p)[i];
 }
 
+// exp(-a) through the hardware base-2 exponential (1 ulp); the rounding error of the product
+// -a * log2(e) is carried separately and folded back in, so the result stays within about 2 ulp for
+// every argument instead of growing with |a|.
+MSLK_AMD_DEVINL float exp_neg(float a) {
+  constexpr float kLog2eHi = 1.44269502162933349609375f, kLog2eLo = 1.925963033500011e-8f, kLn2 = 0.693147182464599609375f;
+  const float na = -a;
+  const float t = na * kLog2eHi;
+  float e = __builtin_fmaf(na, kLog2eHi, -t);
+  e = __builtin_fmaf(na, kLog2eLo, e);
+  const float p = __builtin_amdgcn_exp2f(t);
+  return __builtin_fmaf(p, e * kLn2, p);
+}
+
+// sigmoid through the hardware reciprocal (1 ulp): the convert that follows keeps 3 mantissa bits.
 MSLK_AMD_DEVINL float silu_mul(float a, float b) {
-  const float sig = 1.0f / (1.0f + __builtin_expf(-a));
+  const float sig = __builtin_amdgcn_rcpf(1.0f + exp_neg(a));
   return (a * sig) * b;
 }
 
