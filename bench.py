@@ -319,6 +319,7 @@ def main():
         Nd = Kd = 8192
         wq3, ws3 = mslk_amd.quantize_fp8_row(W.cfg3_weight().to(dev))
         wsets = [wq3.clone() for _ in range(6)]  # 6 x 64 MiB > Infinity Cache
+        wshuf = [mslk_amd.preshuffle_b_mfma(w) for w in wsets]   # the same weights in the pre-shuffled (blocked) layout
         decode = {}
         for Md in (1, 4, 16, 64):
             xd = W.cfg3_activations(Md).to(dev)
@@ -332,17 +333,25 @@ def main():
                 api.quantize(xd, xq3, xs3)
                 api.gemm(xq3, wsets[i % len(wsets)], xs3, ws3, y3)
 
+            def dec_ps_step(i):
+                api.check(api.L.mslk_amd_f8f8_rowwise_preshuffle(xq3.data_ptr(), wshuf[i % len(wshuf)].data_ptr(), xs3.data_ptr(),
+                                                                 ws3.data_ptr(), None, 0, y3.data_ptr(), 0, Md, Nd, Kd, api.stream))
+
             for i in range(12):
                 dec_step(i)
+                dec_ps_step(i)
+            ms_ps = _median_events_ms(dec_ps_step, 60)
             ms = _median_events_ms(dec_step, 60)
             ms_path = _median_events_ms(dec_path_step, 60)
             ms_graph = _graph_ms(dec_step, 60)
             nbytes = Nd * Kd + Md * Kd + 2.0 * Md * Nd + 4.0 * (Md + Nd)
             decode[f"M{Md}"] = {"ms": ms, "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / PEAK_HBM_BPS,
                                 "ms_with_quantize": ms_path, "bytes": nbytes, "ms_graph_replay": ms_graph,
-                                "GBps_graph_replay": nbytes / (ms_graph * 1e-3) / 1e9}
+                                "GBps_graph_replay": nbytes / (ms_graph * 1e-3) / 1e9,
+                                "ms_preshuffled_weights": ms_ps, "GBps_preshuffled_weights": nbytes / (ms_ps * 1e-3) / 1e9,
+                                "frac_hbm_preshuffled_weights": nbytes / (ms_ps * 1e-3) / PEAK_HBM_BPS}
         extras["decode_N8192_K8192"] = decode
-        del wsets
+        del wsets, wshuf
         if args.only == "decode":
             print(json.dumps(extras))
             return

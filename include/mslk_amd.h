@@ -134,6 +134,27 @@ int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scal
                              void* stream);
 
 /*
+ * The dense GEMM on PRE-SHUFFLED weights.  Replaces mslk::gemm::f8f8bf16_rowwise_preshuffle and
+ * f8f8f16_rowwise_preshuffle (reference: csrc/gemm/gemm_ops.cpp:90-93,
+ * csrc/gemm/ck/fp8_rowwise_preshuffle/fp8_rowwise_preshuffle_gemm.hip:93-171).  `wq_shuffled` holds the
+ * [N, K] weights in the blocked order [N/16][K/64][4][16][16 bytes] that ck_preshuffle(wq, 16) /
+ * preshuffle_b_mfma produce (reference: mslk/quantize/shuffle.py:182-246): every 16-row x 64-byte block is
+ * stored as (16-byte k chunk, row, byte), i.e. in the order the 64 lanes of an MFMA operand read it.
+ * Requires N % 16 == 0 and K % 64 == 0; everything else as mslk_amd_f8f8bf16_rowwise.
+ * y_dtype: MSLK_AMD_DTYPE_BF16 or MSLK_AMD_DTYPE_F16.
+ */
+int mslk_amd_f8f8_rowwise_preshuffle(const void* xq, const void* wq_shuffled, const float* x_scale, const float* w_scale,
+                                     const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M, int64_t N,
+                                     int64_t K, void* stream);
+
+/*
+ * Weight re-layout for the entry point above: wq [G, N, K] row-major -> wq_shuffled, the blocked
+ * order applied to each of the G matrices (out of place).  Replaces ck_preshuffle / preshuffle_b_mfma
+ * (reference: mslk/quantize/shuffle.py:182-246).  N % 16 == 0, K % 64 == 0, 16-byte aligned pointers.
+ */
+int mslk_amd_preshuffle_b(const void* wq, void* wq_shuffled, int64_t G, int64_t N, int64_t K, void* stream);
+
+/*
  * Grouped (MoE) rowwise FP8 GEMM over G independent problems given as host arrays of device
  * pointers.  Replaces mslk::gemm::f8f8bf16_rowwise_grouped (TensorList API; reference:
  * csrc/gemm/gemm_ops.cpp:37-38, csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:481-559,586-593).

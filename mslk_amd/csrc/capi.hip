@@ -124,7 +124,7 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
 
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
 
-static int rowwise_impl(const char* op, int out_f16, const void* xq, const void* wq, const float* x_scale,
+static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void* xq, const void* wq, const float* x_scale,
                         const float* w_scale, const void* bias, int bias_dtype, void* y, int64_t M, int64_t N,
                         int64_t K, void* stream) {
   if (M < 0 || N < 0 || K < 0) return fail("%s: negative dimension", op);
@@ -136,8 +136,10 @@ static int rowwise_impl(const char* op, int out_f16, const void* xq, const void*
   if (!y) return fail("%s: null output", op);
   if (K == 0) return check_hip(launch_fill_zero_bf16((uint16_t*)y, M * N, s), "zero fill");
   if (!xq || !wq || !x_scale || !w_scale) return fail("%s: null pointer", op);
+  if (preshuffled && (N % 16 != 0 || K % 64 != 0))
+    return fail("%s: pre-shuffled weights need N %% 16 == 0 and K %% 64 == 0 (got N=%lld, K=%lld)", op, (long long)N, (long long)K);
   GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
-                (int)M, (int)N, (int)K, bias_dtype, out_f16};
+                (int)M, (int)N, (int)K, bias_dtype, out_f16, preshuffled};
   if (skinny_supports(p)) return check_hip(launch_skinny(p, s), "skinny launch");
   if (dense_tiled_supports(p)) return check_hip(launch_dense_tiled(p, s), "tiled launch");
   return check_hip(launch_generic(p, s), "generic launch");
@@ -146,13 +148,32 @@ static int rowwise_impl(const char* op, int out_f16, const void* xq, const void*
 int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                               const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
                               void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
-  return rowwise_impl("f8f8bf16_rowwise", 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+  return rowwise_impl("f8f8bf16_rowwise", 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
 }
 
 int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
                              void* stream) {
-  return rowwise_impl("f8f8f16_rowwise", 1, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+  return rowwise_impl("f8f8f16_rowwise", 1, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+}
+
+int mslk_amd_f8f8_rowwise_preshuffle(const void* xq, const void* wq_shuffled, const float* x_scale, const float* w_scale,
+                                     const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M, int64_t N,
+                                     int64_t K, void* stream) {
+  if (y_dtype != MSLK_AMD_DTYPE_BF16 && y_dtype != MSLK_AMD_DTYPE_F16)
+    return fail("f8f8_rowwise_preshuffle: output dtype code %d is neither bf16 nor fp16", y_dtype);
+  return rowwise_impl(y_dtype == MSLK_AMD_DTYPE_F16 ? "f8f8f16_rowwise_preshuffle" : "f8f8bf16_rowwise_preshuffle",
+                      y_dtype == MSLK_AMD_DTYPE_F16, 1, xq, wq_shuffled, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+}
+
+int mslk_amd_preshuffle_b(const void* wq, void* wq_shuffled, int64_t G, int64_t N, int64_t K, void* stream) {
+  if (G < 0 || N < 0 || K < 0) return fail("preshuffle_b: negative dimension");
+  if (N % 16 != 0 || K % 64 != 0) return fail("preshuffle_b needs N %% 16 == 0 and K %% 64 == 0, got N=%lld K=%lld", (long long)N, (long long)K);
+  if (G == 0 || N == 0 || K == 0) return 0;
+  if (!wq || !wq_shuffled) return fail("preshuffle_b: null pointer");
+  if (wq == wq_shuffled) return fail("preshuffle_b: the permutation cannot run in place");
+  if (reinterpret_cast<uintptr_t>(wq) % 16 || reinterpret_cast<uintptr_t>(wq_shuffled) % 16) return fail("preshuffle_b: pointers must be 16-byte aligned");
+  return check_hip(launch_preshuffle_b(wq, wq_shuffled, G, N, K, (hipStream_t)stream), "preshuffle_b launch");
 }
 
 int mslk_amd_f8f8bf16_rowwise_grouped(int G, const void* const* xq, const void* const* wq,
@@ -181,7 +202,7 @@ int mslk_amd_f8f8bf16_rowwise_grouped(int G, const void* const* xq, const void* 
     }
     if (!xq[g] || !wq[g] || !x_scale[g] || !w_scale[g]) return fail("f8f8bf16_rowwise_grouped: null pointer in group %d", g);
     GemmProblem p{(const uint8_t*)xq[g], (const uint8_t*)wq[g], x_scale[g], w_scale[g], nullptr, (uint16_t*)y[g],
-                  (int)M[g], (int)N[g], (int)K[g], 0, 0};
+                  (int)M[g], (int)N[g], (int)K[g], 0, 0, 0};
     if (!dense_tiled_supports(p)) {  // odd K or alignment: per-group fallback
       if (int rc = check_hip(launch_generic(p, s), "generic launch")) return rc;
       continue;

@@ -24,14 +24,14 @@ MSLK_AMD_DEVINL bool map_tile(int bid, int tiles_m, int tiles_n, int& tm, int& t
   return true;
 }
 
-template <typename TS, int BIAS>
+template <typename TS, int BIAS, bool PS>
 __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int BM = TS::kBM, BN = TS::kBN;
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
   int tm, tn;
   if (!map_tile(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
-  GemmTile<TS, BIAS> tile;
+  GemmTile<TS, BIAS, PS> tile;
   tile.out_f16 = p.out_f16;
   const void* bias = nullptr;
   if constexpr (BIAS == 1) bias = reinterpret_cast<const float*>(p.bias) + n0;
@@ -40,16 +40,16 @@ __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p
            p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K);
 }
 
-template <typename TS>
+template <typename TS, bool PS>
 hipError_t launch_tiled_shape(const GemmProblem& p, hipStream_t s) {
   constexpr int BM = TS::kBM, BN = TS::kBN;
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const int grid = ((ntiles + kXcds - 1) / kXcds) * kXcds;
   switch (p.bias_dtype) {
-    case 0: dense_tiled_kernel<TS, 0><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
-    case 1: dense_tiled_kernel<TS, 1><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
-    default: dense_tiled_kernel<TS, 2><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    case 0: dense_tiled_kernel<TS, 0, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    case 1: dense_tiled_kernel<TS, 1, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    default: dense_tiled_kernel<TS, 2, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
   }
   return hipGetLastError();
 }
@@ -60,14 +60,40 @@ __global__ __launch_bounds__(256) void generic_kernel(GemmProblem p) {
   if (idx >= (int64_t)p.M * p.N) return;
   const int m = (int)(idx / p.N), n = (int)(idx % p.N);
   const uint8_t* a = p.xq + (int64_t)m * p.K;
-  const uint8_t* b = p.wq + (int64_t)n * p.K;
   float acc = 0.f;
-  for (int k = 0; k < p.K; ++k)
-    acc += __builtin_amdgcn_cvt_f32_fp8((int)a[k], 0) * __builtin_amdgcn_cvt_f32_fp8((int)b[k], 0);
+  if (p.w_preshuffled) {
+    // element (n, k) of the blocked layout [N/16][K/64][4][16][16]
+    const uint8_t* b = p.wq + (int64_t)(n >> 4) * 16 * p.K + (n & 15) * 16;
+    for (int k = 0; k < p.K; ++k)
+      acc += __builtin_amdgcn_cvt_f32_fp8((int)a[k], 0) *
+             __builtin_amdgcn_cvt_f32_fp8((int)b[(int64_t)(k >> 6) * 1024 + ((k >> 4) & 3) * 256 + (k & 15)], 0);
+  } else {
+    const uint8_t* b = p.wq + (int64_t)n * p.K;
+    for (int k = 0; k < p.K; ++k)
+      acc += __builtin_amdgcn_cvt_f32_fp8((int)a[k], 0) * __builtin_amdgcn_cvt_f32_fp8((int)b[k], 0);
+  }
   float v = (acc * p.xs[m]) * p.ws[n];
   if (p.bias_dtype == 1) v += reinterpret_cast<const float*>(p.bias)[n];
   else if (p.bias_dtype == 2) v += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]);
   p.y[idx] = (uint16_t)f32_to_out_bits(v, p.out_f16);
+}
+
+// Row-major [G, N, K] -> blocked [G][N/16][K/64][4][16][16 B] (reference: ck_preshuffle / preshuffle_b_mfma,
+// mslk/quantize/shuffle.py:182-246).  A pure permutation of 16-byte chunks; one lane moves one chunk, and
+// the lanes of a wave write 1 KiB contiguous while reading 16 rows x 64 bytes.
+__global__ __launch_bounds__(256) void preshuffle_b_kernel(const v4i* __restrict__ src, v4i* __restrict__ dst, int64_t chunks,
+                                                           int K) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  const int kblocks = K >> 6;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += stride) {
+    // destination chunk c = ((group * kblocks + kb) * 4 + klane) * 16 + nlane   (group counts 16-row groups over G * N / 16)
+    const int nlane = (int)(c & 15), klane = (int)((c >> 4) & 3);
+    const int64_t blk = c >> 6;
+    const int64_t group = blk / kblocks;
+    const int kb = (int)(blk - group * kblocks);
+    const int64_t row = group * 16 + nlane;
+    dst[c] = src[row * (K >> 4) + kb * 4 + klane];
+  }
 }
 
 __global__ void fill_zero_kernel(uint16_t* y, int64_t n) {
@@ -78,6 +104,7 @@ __global__ void fill_zero_kernel(uint16_t* y, int64_t n) {
 }  // namespace
 
 bool dense_tiled_supports(const GemmProblem& p) {
+  if (p.w_preshuffled && (p.N % 16 != 0 || p.K % 64 != 0)) return false;   // the blocked layout itself needs this
   return p.K % 16 == 0 && p.K >= 16 && (int64_t)256 * p.K < (int64_t(1) << 32) &&
          reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(p.y) % 16 == 0;
@@ -87,13 +114,26 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (!dense_tiled_supports(p)) return hipErrorInvalidValue;
   // 256 x 256 tiles once they give every CU work; 128 x 128 below that.
   const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
-  if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>>(p, s);
-  return launch_tiled_shape<TileShape<128, 128>>(p, s);
+  if (p.w_preshuffled) {
+    if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
+    return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
+  }
+  if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  return launch_tiled_shape<TileShape<128, 128>, false>(p, s);
 }
 
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s) {
   const int64_t total = (int64_t)p.M * p.N;
   generic_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(p);
+  return hipGetLastError();
+}
+
+hipError_t launch_preshuffle_b(const void* src, void* dst, int64_t G, int64_t N, int64_t K, hipStream_t s) {
+  const int64_t chunks = G * N * (K / 16);
+  if (chunks <= 0) return hipSuccess;
+  const int64_t want = (chunks + 255) / 256;
+  preshuffle_b_kernel<<<(unsigned)(want > 65536 ? 65536 : want), 256, 0, s>>>(static_cast<const v4i*>(src), static_cast<v4i*>(dst),
+                                                                              chunks, (int)K);
   return hipGetLastError();
 }
 

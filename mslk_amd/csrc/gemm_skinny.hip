@@ -37,7 +37,10 @@ MSLK_AMD_DEVINL v4i load16_stream(const uint8_t* p) {
 
 // One batch: the loads of U K-steps of this wave (steps kt0, kt0 + 8, ...), then their MFMAs.
 // CHECKED = false is the fast path: every step lies fully inside K, so no lane is predicated.
-template <int MT, int NT, int U, int kWaves, bool CHECKED>
+// PS: the weights are in the blocked layout [N/16][K/64][4][16][16 B]; wp[tn] then points at this
+// lane's 16 bytes of the first block of its row group, and the two halves of a K step are the next
+// two 1 KiB blocks, each read by the wave as one contiguous KiB.
+template <int MT, int NT, int U, int kWaves, bool CHECKED, bool PS = false>
 MSLK_AMD_DEVINL void skinny_batch(const uint8_t* const (&wp)[NT], const uint8_t* const (&xp)[MT], int kt0, int K, int g,
                                   v4f (&acc)[NT][MT]) {
   v8i wf[U][NT], xf[U][MT];
@@ -48,12 +51,13 @@ MSLK_AMD_DEVINL void skinny_batch(const uint8_t* const (&wp)[NT], const uint8_t*
 #pragma unroll
     for (int tn = 0; tn < NT; ++tn) {
       v4i lo, hi;
+      const int64_t w0 = PS ? (int64_t)k0 * 16 : k0, w1 = PS ? w0 + 1024 : w0 + 64;
       if constexpr (CHECKED) {
-        lo = load16_or_zero(wp[tn] + k0, ok0);
-        hi = load16_or_zero(wp[tn] + k0 + 64, ok1);
+        lo = load16_or_zero(wp[tn] + w0, ok0);
+        hi = load16_or_zero(wp[tn] + w1, ok1);
       } else {
-        lo = load16_stream(wp[tn] + k0);
-        hi = load16_stream(wp[tn] + k0 + 64);
+        lo = load16_stream(wp[tn] + w0);
+        hi = load16_stream(wp[tn] + w1);
       }
       wf[u][tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
@@ -79,7 +83,7 @@ MSLK_AMD_DEVINL void skinny_batch(const uint8_t* const (&wp)[NT], const uint8_t*
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[u][tn], xf[u][tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
 }
 
-template <int MT, int NT, int U, int kWaves, int BIAS>
+template <int MT, int NT, int U, int kWaves, int BIAS, bool PS>
 __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
   __shared__ float red[kWaves][NT][MT][256];
   const int lane = threadIdx.x & 63;
@@ -93,8 +97,13 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
   const uint8_t* wp[NT];
 #pragma unroll
   for (int tn = 0; tn < NT; ++tn) {
-    const int row = n0 + tn * 16 + i;
-    wp[tn] = p.wq + (int64_t)(row < p.N ? row : p.N - 1) * K + g * 16;
+    if constexpr (PS) {
+      const int group = (n0 >> 4) + tn, groups = p.N >> 4;
+      wp[tn] = p.wq + (int64_t)(group < groups ? group : groups - 1) * 16 * K + lane * 16;
+    } else {
+      const int row = n0 + tn * 16 + i;
+      wp[tn] = p.wq + (int64_t)(row < p.N ? row : p.N - 1) * K + g * 16;
+    }
   }
   const uint8_t* xp[MT];
 #pragma unroll
@@ -132,10 +141,10 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
   int kt0 = wave;
   if (K % (kWaves * kStep) == 0) {
     // every wave owns the same number of complete steps: unpredicated batches
-    for (; kt0 + (U - 1) * kWaves < KT; kt0 += kWaves * U) skinny_batch<MT, NT, U, kWaves, false>(wp, xp, kt0, K, g, acc);
-    for (; kt0 < KT; kt0 += kWaves) skinny_batch<MT, NT, 1, kWaves, false>(wp, xp, kt0, K, g, acc);
+    for (; kt0 + (U - 1) * kWaves < KT; kt0 += kWaves * U) skinny_batch<MT, NT, U, kWaves, false, PS>(wp, xp, kt0, K, g, acc);
+    for (; kt0 < KT; kt0 += kWaves) skinny_batch<MT, NT, 1, kWaves, false, PS>(wp, xp, kt0, K, g, acc);
   } else {
-    for (; kt0 < KT; kt0 += kWaves * 2) skinny_batch<MT, NT, 2, kWaves, true>(wp, xp, kt0, K, g, acc);
+    for (; kt0 < KT; kt0 += kWaves * 2) skinny_batch<MT, NT, 2, kWaves, true, PS>(wp, xp, kt0, K, g, acc);
   }
 
 #pragma unroll
@@ -162,13 +171,13 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
   }
 }
 
-template <int MT, int NT, int U, int kWaves = 8>
+template <int MT, int NT, int U, bool PS = false, int kWaves = 8>
 hipError_t launch_cfg(const GemmProblem& p, hipStream_t s) {
   const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
   switch (p.bias_dtype) {
-    case 0: skinny_kernel<MT, NT, U, kWaves, 0><<<grid, kWaves * 64, 0, s>>>(p); break;
-    case 1: skinny_kernel<MT, NT, U, kWaves, 1><<<grid, kWaves * 64, 0, s>>>(p); break;
-    default: skinny_kernel<MT, NT, U, kWaves, 2><<<grid, kWaves * 64, 0, s>>>(p); break;
+    case 0: skinny_kernel<MT, NT, U, kWaves, 0, PS><<<grid, kWaves * 64, 0, s>>>(p); break;
+    case 1: skinny_kernel<MT, NT, U, kWaves, 1, PS><<<grid, kWaves * 64, 0, s>>>(p); break;
+    default: skinny_kernel<MT, NT, U, kWaves, 2, PS><<<grid, kWaves * 64, 0, s>>>(p); break;
   }
   return hipGetLastError();
 }
@@ -189,10 +198,15 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 MSLK_AMD_DEVINL int row_swz(int row) { return (row & 7) ^ ((row >> 3) & 1); }
 
-template <int MT, int NT, int U, int BIAS>
+//
+// PS (pre-shuffled weights, blocked layout [N/16][K/64][4][16][16 B]): a weight fragment is two
+// contiguous KiB blocks, so the weights go global -> VGPR with full-line requests and only the
+// activations are staged.
+template <int MT, int NT, int U, int BIAS, bool PS = false>
 __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
   constexpr int kWaves = 8;
-  constexpr int XBUF = U * (MT + NT) * 2048;                // bytes of staged operands per wave
+  constexpr int WT = PS ? 0 : NT;                           // weight tiles staged in LDS per step
+  constexpr int XBUF = (U * (MT + WT) * 2048 > NT * MT * 1024) ? U * (MT + WT) * 2048 : NT * MT * 1024;
   static_assert(XBUF >= NT * MT * 1024, "the reduction slot of a wave lives inside its staging buffer");
   __shared__ __attribute__((aligned(1024))) char lds[kWaves * XBUF];
   const int lane = threadIdx.x & 63;
@@ -205,14 +219,18 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
   // weight rows of this workgroup, as DMA source offsets (same lane -> (row, chunk) map as the activations)
   uint32_t w_off[NT][2];
   const uint8_t* w_base = p.wq + (int64_t)n0 * K;
+  const uint8_t* wps[NT];   // PS: this lane's 16 bytes of the first block of each row group
 #pragma unroll
-  for (int tn = 0; tn < NT; ++tn)
+  for (int tn = 0; tn < NT; ++tn) {
+    const int group = (n0 >> 4) + tn, groups = p.N >> 4;
+    wps[tn] = p.wq + (int64_t)(group < groups ? group : groups - 1) * 16 * K + lane * 16;
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int r = 8 * h + (lane >> 3);
       const int row = tn * 16 + r;
       w_off[tn][h] = (uint32_t)(n0 + row < p.N ? row : p.N - 1 - n0) * (uint32_t)K + (((lane & 7) ^ row_swz(r)) << 4);
     }
+  }
   // DMA source offsets: load h (0 / 1) of m-tile tm covers rows tm*16 + 8h + (lane >> 3); lane fetches the
   // logical 16-byte chunk that belongs at physical position (lane & 7) of its swizzled LDS row.
   uint32_t x_off[MT][2];
@@ -255,17 +273,25 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
   const int KT = K / kStep;   // K % (8 * 128) == 0: every wave owns KT / 8 complete steps
   for (int kt0 = wave; kt0 < KT; kt0 += kWaves * U) {
     // Weights first: their HBM requests must not queue behind the (L2-resident) activation traffic.
+    v8i wreg[U][NT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int kt = kt0 + u * kWaves;
       if (kt < KT) {           // wave-uniform
         const int k0 = kt * kStep;
 #pragma unroll
-        for (int tn = 0; tn < NT; ++tn)
+        for (int tn = 0; tn < NT; ++tn) {
+          if constexpr (PS) {
+            const v4i lo = load16_stream(wps[tn] + (int64_t)k0 * 16);
+            const v4i hi = load16_stream(wps[tn] + (int64_t)k0 * 16 + 1024);
+            wreg[u][tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          } else {
 #pragma unroll
-          for (int h = 0; h < 2; ++h)
-            __builtin_amdgcn_global_load_lds((gbl_ptr_t)(w_base + k0 + w_off[tn][h]),
-                                             (lds_ptr_t)(xbuf + ((u * (MT + NT) + MT + tn) * 2 + h) * 1024), 16, 0, 0);
+            for (int h = 0; h < 2; ++h)
+              __builtin_amdgcn_global_load_lds((gbl_ptr_t)(w_base + k0 + w_off[tn][h]),
+                                               (lds_ptr_t)(xbuf + ((u * (MT + WT) + MT + tn) * 2 + h) * 1024), 16, 0, 0);
+          }
+        }
       }
     }
 #pragma unroll
@@ -278,7 +304,7 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
 #pragma unroll
           for (int h = 0; h < 2; ++h)
             __builtin_amdgcn_global_load_lds((gbl_ptr_t)(p.xq + k0 + x_off[tm][h]),
-                                             (lds_ptr_t)(xbuf + ((u * (MT + NT) + tm) * 2 + h) * 1024), 16, 0, 0);
+                                             (lds_ptr_t)(xbuf + ((u * (MT + WT) + tm) * 2 + h) * 1024), 16, 0, 0);
       }
     }
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's DMA has landed in its private buffer
@@ -288,14 +314,18 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
         v8i wf[NT];
 #pragma unroll
         for (int tn = 0; tn < NT; ++tn) {
-          const char* wt = xbuf + (u * (MT + NT) + MT + tn) * 2048;
-          const v4i lo = *reinterpret_cast<const v4i*>(wt + xr0);
-          const v4i hi = *reinterpret_cast<const v4i*>(wt + xr1);
-          wf[tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          if constexpr (PS) {
+            wf[tn] = wreg[u][tn];
+          } else {
+            const char* wt = xbuf + (u * (MT + WT) + MT + tn) * 2048;
+            const v4i lo = *reinterpret_cast<const v4i*>(wt + xr0);
+            const v4i hi = *reinterpret_cast<const v4i*>(wt + xr1);
+            wf[tn] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+          }
         }
 #pragma unroll
         for (int tm = 0; tm < MT; ++tm) {
-          const char* xt = xbuf + (u * (MT + NT) + tm) * 2048;
+          const char* xt = xbuf + (u * (MT + WT) + tm) * 2048;
           const v4i lo = *reinterpret_cast<const v4i*>(xt + xr0);
           const v4i hi = *reinterpret_cast<const v4i*>(xt + xr1);
           const v8i xf = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
@@ -333,13 +363,13 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
   }
 }
 
-template <int MT, int NT, int U>
+template <int MT, int NT, int U, bool PS = false>
 hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
   const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
   switch (p.bias_dtype) {
-    case 0: skinny_lds_kernel<MT, NT, U, 0><<<grid, 512, 0, s>>>(p); break;
-    case 1: skinny_lds_kernel<MT, NT, U, 1><<<grid, 512, 0, s>>>(p); break;
-    default: skinny_lds_kernel<MT, NT, U, 2><<<grid, 512, 0, s>>>(p); break;
+    case 0: skinny_lds_kernel<MT, NT, U, 0, PS><<<grid, 512, 0, s>>>(p); break;
+    case 1: skinny_lds_kernel<MT, NT, U, 1, PS><<<grid, 512, 0, s>>>(p); break;
+    default: skinny_lds_kernel<MT, NT, U, 2, PS><<<grid, 512, 0, s>>>(p); break;
   }
   return hipGetLastError();
 }
@@ -347,12 +377,26 @@ hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
 }  // namespace
 
 bool skinny_supports(const GemmProblem& p) {
+  if (p.w_preshuffled && (p.N % 16 != 0 || p.K % 64 != 0)) return false;
   return p.M >= 1 && p.M <= 64 && p.K % 16 == 0 && p.K >= 16 &&
          reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0;
 }
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
   if (!skinny_supports(p)) return hipErrorInvalidValue;
+  if (p.w_preshuffled && p.K % (8 * kStep) == 0 && p.M > 4) {
+    // weights straight into registers (contiguous KiB blocks), activations through LDS
+    if (p.M <= 16) return launch_lds<1, 2, 2, true>(p, s);
+    if (p.M <= 32) return launch_lds<2, 2, 1, true>(p, s);
+    if (p.M <= 48) return launch_lds<3, 2, 1, true>(p, s);
+    return launch_lds<4, 2, 1, true>(p, s);
+  }
+  if (p.w_preshuffled) {   // weight fragments are contiguous KiB blocks: straight into registers
+    if (p.M <= 16) return launch_cfg<1, 1, 8, true>(p, s);
+    if (p.M <= 32) return launch_cfg<2, 2, 4, true>(p, s);
+    if (p.M <= 48) return launch_cfg<3, 2, 4, true>(p, s);
+    return launch_cfg<4, 2, 4, true>(p, s);
+  }
   if (p.K % (8 * kStep) == 0) {   // both operands through LDS, all global traffic in full lines
     if (p.M <= 16) return launch_lds<1, 1, 4>(p, s);
     if (p.M <= 32) return launch_lds<2, 1, 1>(p, s);

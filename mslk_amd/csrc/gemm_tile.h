@@ -63,7 +63,12 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
 }
 
 
-template <typename TS, int BIAS>
+// PS (pre-shuffled weights): WQ arrives in the blocked layout [N/16][K/64][4][16][16 B] -- each
+// 16-row x 64-byte block stored as (k chunk, row, 16 bytes), the order in which the 64 lanes of an
+// MFMA operand read it (reference: mslk/quantize/shuffle.py:182-246).  One DMA then moves one block
+// (1 KiB contiguous in HBM and in LDS), the WQ fragment read is lane-linear, and both operands give
+// lane (i, g) the k bytes [16 g, 16 g + 16) and [64 + 16 g, 64 + 16 g + 16) of row i.
+template <typename TS, int BIAS, bool PS = false>
 struct GemmTile {
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
@@ -87,10 +92,18 @@ struct GemmTile {
     }
 #pragma unroll
     for (int i = 0; i < TS::LB; ++i) {
-      const int row = (wave * TS::LB + i) * 8 + (lane >> 3);
-      const int chunk = (lane & 7) ^ lds_swz(row);
-      const int rc = row < rows_b ? row : rows_b - 1;
-      b_off[i] = (uint32_t)rc * ld + chunk * 16;
+      if constexpr (PS) {
+        // load q of the stage = block (16-row group q / 2, 64-byte half q % 2); edge tiles re-read the last group
+        const int q = wave * TS::LB + i;
+        const int groups = rows_b >> 4;
+        const int nb = (q >> 1) < groups ? (q >> 1) : groups - 1;
+        b_off[i] = (uint32_t)nb * 16u * ld + (q & 1) * 1024 + lane * 16;
+      } else {
+        const int row = (wave * TS::LB + i) * 8 + (lane >> 3);
+        const int chunk = (lane & 7) ^ lds_swz(row);
+        const int rc = row < rows_b ? row : rows_b - 1;
+        b_off[i] = (uint32_t)rc * ld + chunk * 16;
+      }
     }
   }
 
@@ -102,7 +115,8 @@ struct GemmTile {
     dma16(a_base + k0 + a_off[i], stage + (wave_id() * TS::LA + i) * 1024);
   }
   MSLK_AMD_DEVINL void issue_b(char* stage, int k0, int i) {
-    dma16(b_base + k0 + b_off[i], stage + TS::A_BYTES + (wave_id() * TS::LB + i) * 1024);
+    // pre-shuffled: the K step at byte k0 starts 16 rows x k0 bytes into the row group
+    dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], stage + TS::A_BYTES + (wave_id() * TS::LB + i) * 1024);
   }
 
   // All DMA loads of a full K step (128 valid bytes per row) starting at byte k0 into `stage`.
@@ -130,24 +144,38 @@ struct GemmTile {
       const int row = (wave * TS::LB + i) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swz(row);
       char* dst = stage + TS::A_BYTES + (wave * TS::LB + i) * 1024;
-      if (chunk * 16 < k_valid) dma16(b_base + k0 + b_off[i], dst);
+      const bool valid = PS ? ((wave * TS::LB + i) & 1) * 64 < k_valid : chunk * 16 < k_valid;
+      if (valid) dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], dst);
       else *reinterpret_cast<uint4*>(dst + lane * 16) = make_uint4(0, 0, 0, 0);
     }
   }
 
   // LDS byte offsets of this lane's two 16-byte halves of an MFMA operand fragment, relative to the
-  // first row of the fragment: lane (i = l & 15, g = l >> 4) reads logical chunks 2g and 2g + 1 of row i.
+  // first row of the fragment: lane (i = l & 15, g = l >> 4) reads logical chunks 2g and 2g + 1 of row i
+  // (chunks g and g + 4 when the weights are pre-shuffled, whose blocks fix that k assignment).
   struct FragOff { int off0, off1; };
   MSLK_AMD_DEVINL static FragOff frag_off() {
     const int lane = threadIdx.x & 63;
     const int i = lane & 15, g = lane >> 4;
     const int s = lds_swz(i);
-    return FragOff{i * kBK + (((2 * g) ^ s) << 4), i * kBK + (((2 * g + 1) ^ s) << 4)};
+    const int c0 = PS ? g : 2 * g, c1 = PS ? g + 4 : 2 * g + 1;
+    return FragOff{i * kBK + ((c0 ^ s) << 4), i * kBK + ((c1 ^ s) << 4)};
   }
   MSLK_AMD_DEVINL static v8i load_frag(const char* tile, int t, FragOff fo) {
     const v4i lo = *reinterpret_cast<const v4i*>(tile + t * 16 * kBK + fo.off0);
     const v4i hi = *reinterpret_cast<const v4i*>(tile + t * 16 * kBK + fo.off1);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  }
+  // WQ fragment t of the wave: as load_frag, or lane-linear out of the two 1 KiB blocks of row group t.
+  MSLK_AMD_DEVINL static v8i load_frag_b(const char* tile, int t, FragOff fo) {
+    if constexpr (PS) {
+      const char* blk = tile + t * 2048 + (threadIdx.x & 63) * 16;
+      const v4i lo = *reinterpret_cast<const v4i*>(blk);
+      const v4i hi = *reinterpret_cast<const v4i*>(blk + 1024);
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    } else {
+      return load_frag(tile, t, fo);
+    }
   }
   MSLK_AMD_DEVINL static const char* a_tile_of(const char* stage) {
     return stage + (wave_id() / TS::WN) * (TS::kBM / TS::WM) * kBK;
@@ -158,7 +186,7 @@ struct GemmTile {
   // First fragments of a K step: all XQ fragments and WQ fragment 0.
   MSLK_AMD_DEVINL void load_first_frags(const char* stage, v8i (&xf)[TS::FM], v8i& wf0) {
     const FragOff fo = frag_off();
-    wf0 = load_frag(b_tile_of(stage), 0, fo);
+    wf0 = load_frag_b(b_tile_of(stage), 0, fo);
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) xf[tm] = load_frag(a_tile_of(stage), tm, fo);
   }
@@ -195,7 +223,7 @@ struct GemmTile {
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) {
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
-        if (tm == 0) wf_next = load_frag(b_tile, tn + 1, fo);
+        if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
         if constexpr (DMA) {
           const int d = tm - (TS::FM - NDMA);
           if (tn < HALF && d >= 0) {
@@ -210,7 +238,7 @@ struct GemmTile {
     }
     if constexpr (NEXT) {
       __syncthreads();  // s_waitcnt vmcnt(0) lgkmcnt(0); s_barrier
-      wf0 = load_frag(b_tile_of(nxt), 0, fo);
+      wf0 = load_frag_b(b_tile_of(nxt), 0, fo);
     }
     const char* a_next = a_tile_of(nxt);
 #pragma unroll

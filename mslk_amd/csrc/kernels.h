@@ -13,6 +13,8 @@ hipError_t launch_quantize_fp8_row(const void* x, int dtype, int64_t rows, int64
                                    hipStream_t s);
 hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out,
                                      hipStream_t s);
+// WQ [G, N, K] row-major -> the blocked layout the *_preshuffle GEMMs read (N % 16 == 0, K % 64 == 0).
+hipError_t launch_preshuffle_b(const void* src, void* dst, int64_t G, int64_t N, int64_t K, hipStream_t s);
 hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t s);
 
 // Fused producers of quantized activations (fused_quant.hip).
@@ -52,6 +54,7 @@ struct GemmProblem {
   int M, N, K;
   int bias_dtype;     // 0 none, 1 fp32, 2 bf16
   int out_f16;        // 0: Y is bf16, 1: Y is fp16
+  int w_preshuffled;  // 1: WQ is in the blocked layout [N/16][K/64][4][16][16 B] (N % 16 == 0, K % 64 == 0)
 };
 
 // Shape classes; each returns hipErrorInvalidValue when the shape is outside what it supports.

@@ -1,6 +1,6 @@
 """`torch.ops.mslk.*` rowwise FP8 GEMM operators backed by the gfx950 HIP kernels.
 
-The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-44,88-89,95-96), so callers written
+The schema strings are the reference's (csrc/gemm/gemm_ops.cpp:31-44,88-96), so callers written
 against `torch.ops.mslk.f8f8bf16_rowwise` etc. run unchanged.  When the reference's own library has
 already defined a schema, only the GPU ("CUDA" dispatch key) kernel is replaced -- the same seam
 the reference's Python kernels use (mslk/gemm/flydsl/preshuffle_gemm.py:433-475).
@@ -27,6 +27,8 @@ _SCHEMAS = {
     "f8f8bf16_rowwise": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
     "f8f8bf16_rowwise_out": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor(a!) output, Tensor? bias=None, bool use_fast_accum=True) -> ()",
     "f8f8f16_rowwise": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
+    "f8f8bf16_rowwise_preshuffle": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
+    "f8f8f16_rowwise_preshuffle": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True) -> Tensor",
     "f8f8bf16_rowwise_grouped": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor[]",
     "f8f8bf16_rowwise_grouped_cat": "(Tensor[] XQ, Tensor[] WQ, Tensor[] x_scale, Tensor[] w_scale) -> Tensor",
     "f8f8bf16_rowwise_grouped_stacked": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor M_sizes) -> Tensor",
@@ -74,7 +76,8 @@ def _bias_args(bias: Optional[torch.Tensor], N: int, device: torch.device):
     return b.data_ptr(), (1 if b.dtype == torch.float32 else 2), b
 
 
-def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, out_dtype=torch.bfloat16):
+def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, out_dtype=torch.bfloat16,
+                  preshuffled=False):
     _check(XQ.dtype == WQ.dtype, f"XQ and WQ dtypes must match, got {XQ.dtype} vs {WQ.dtype}")
     _check(XQ.dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ.dtype}")
     _check(x_scale.dtype == torch.float32 and w_scale.dtype == torch.float32, "Scales must be float32.")
@@ -110,6 +113,13 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, o
     xs = x_scale.contiguous()
     ws = w_scale.contiguous()
     bias_ptr, bias_code, _keep = _bias_args(bias, N, XQ.device)
+    if preshuffled:
+        _check(N % 16 == 0 and K % 64 == 0, f"pre-shuffled weights need N % 16 == 0 and K % 64 == 0, got N={N} K={K}")
+        with _on_device(XQ.device):
+            _lib.check(_lib.lib().mslk_amd_f8f8_rowwise_preshuffle(
+                XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
+                1 if out_dtype == torch.float16 else 0, M, N, K, _stream_ptr(XQ.device)))
+        return Y
     with _on_device(XQ.device):
         if out_dtype == torch.float16:
             _lib.check(_lib.lib().mslk_amd_f8f8f16_rowwise(
@@ -133,6 +143,42 @@ def f8f8bf16_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_a
 def f8f8f16_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
     """Same GEMM with an fp16 result (fp8fp8fp16_rowwise_gemm.hip:66-133)."""
     return _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, None, torch.float16)
+
+
+def f8f8bf16_rowwise_preshuffle(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
+    """f8f8bf16_rowwise on weights pre-shuffled by `ck_preshuffle(wq, 16)` / `preshuffle_b_mfma(wq)`
+    (fp8_rowwise_preshuffle_gemm.hip:93-171)."""
+    return _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, None, torch.bfloat16, True)
+
+
+def f8f8f16_rowwise_preshuffle(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
+    """fp16-output variant.  (The reference registers its bf16 function under this name too,
+    gemm_ops.cpp:145; the schema and the fp16 wrapper at fp8_rowwise_preshuffle_gemm.hip:160-171 say fp16.)"""
+    return _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, None, torch.float16, True)
+
+
+def preshuffle_b_mfma(src: torch.Tensor) -> torch.Tensor:
+    """FP8 weights [N, K] or [G, N, K] -> the blocked order [N/16][K/64][4][16][16 B] the *_preshuffle GEMMs
+    read (mslk/quantize/shuffle.py:208-246).  Same shape and dtype as `src`; out of place."""
+    _check(src.is_cuda and src.is_contiguous(), "preshuffle_b_mfma: src must be a contiguous GPU tensor")
+    _check(src.element_size() == 1 and src.dim() in (2, 3), "preshuffle_b_mfma: src must be an 8-bit [N, K] or [G, N, K] tensor")
+    N, K = src.shape[-2], src.shape[-1]
+    if N % 16 or K % 64:
+        raise ValueError(f"preshuffle_b_mfma needs N % 16 == 0 and K % 64 == 0, got N={N} K={K}")
+    G = src.shape[0] if src.dim() == 3 else 1
+    dst = torch.empty_like(src)
+    if src.numel():
+        with _on_device(src.device):
+            _lib.check(_lib.lib().mslk_amd_preshuffle_b(src.data_ptr(), dst.data_ptr(), G, N, K, _stream_ptr(src.device)))
+    return dst
+
+
+def ck_preshuffle(src: torch.Tensor, NXdl: int = 16) -> torch.Tensor:
+    """Reference name for the same re-layout of one [N, K] matrix (mslk/quantize/shuffle.py:182-205);
+    only the 16-row wave tile the GEMM reads is supported."""
+    _check(NXdl == 16, "ck_preshuffle: only NXdl = 16 is supported")
+    _check(src.dim() == 2, "ck_preshuffle: src must be [N, K]")
+    return preshuffle_b_mfma(src)
 
 
 def _check_grouped(XQ: Sequence[torch.Tensor], WQ, x_scale, w_scale):
@@ -377,6 +423,8 @@ _IMPLS = {
     "f8f8bf16_rowwise": f8f8bf16_rowwise,
     "f8f8bf16_rowwise_out": f8f8bf16_rowwise_out,
     "f8f8f16_rowwise": f8f8f16_rowwise,
+    "f8f8bf16_rowwise_preshuffle": f8f8bf16_rowwise_preshuffle,
+    "f8f8f16_rowwise_preshuffle": f8f8f16_rowwise_preshuffle,
     "f8f8bf16_rowwise_grouped": f8f8bf16_rowwise_grouped,
     "f8f8bf16_rowwise_grouped_cat": f8f8bf16_rowwise_grouped_cat,
     "f8f8bf16_rowwise_grouped_stacked": f8f8bf16_rowwise_grouped_stacked,
@@ -432,6 +480,8 @@ _FAKES = {
     "f8f8bf16_rowwise": _fake_rowwise,
     "f8f8bf16_rowwise_out": _fake_rowwise_out,
     "f8f8f16_rowwise": _fake_rowwise_f16,
+    "f8f8bf16_rowwise_preshuffle": _fake_rowwise,
+    "f8f8f16_rowwise_preshuffle": _fake_rowwise_f16,
     "f8f8bf16_rowwise_grouped": _fake_grouped,
     "f8f8bf16_rowwise_grouped_cat": _fake_grouped_cat,
     "f8f8bf16_rowwise_grouped_stacked": _fake_grouped_stacked,

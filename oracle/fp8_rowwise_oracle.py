@@ -13,6 +13,7 @@ Every function restates, in plain CPU torch, the arithmetic of one reference fun
   grouped_*               test/gemm/triton/grouped_gemm_test.py:116-121, bench/gemm/gemm_ops.py:632-644
   quantize_fp8_row_jagged mslk/quantize/triton/fp8_quantize.py:123-129,236-243
   dequantize_fp8_row[_bf16] mslk/quantize/triton/fp8_quantize.py:1060-1113
+  preshuffle_b            mslk/quantize/shuffle.py:182-246
   quantize_rows_saturating, silu_mul_quant, gather_scale_quant_dense_tokens
                           mslk/moe/activation.py:232-300, mslk/moe/gather_scatter.py:545-640
 
@@ -124,6 +125,19 @@ def gather_scale_quant_dense_tokens(x: torch.Tensor, token_indices: torch.Tensor
     t, e = token_indices.to(torch.int64), expert_indices.to(torch.int64)
     y = x[t].to(torch.float32) * scores[t, e].to(torch.float32)[:, None]
     return quantize_rows_saturating(y, scale_ub)
+
+
+def preshuffle_b(src: torch.Tensor) -> torch.Tensor:
+    """Blocked weight layout of the reference's pre-shuffled GEMMs (mslk/quantize/shuffle.py:182-246):
+    the trailing [N, K] is cut into 16-row x 64-column blocks, (N/16, 16, K/64, 4, 16), and stored in
+    the order (N/16, K/64, 4, 16, 16) -- block, 16-byte k chunk, row, byte.  Same shape as src."""
+    N, K = src.shape[-2], src.shape[-1]
+    assert N % 16 == 0 and K % 64 == 0
+    lead = src.shape[:-2]
+    v = src.reshape(*lead, N // 16, 16, K // 64, 4, 16)
+    nd = v.dim()
+    v = v.permute(*range(nd - 5), nd - 5, nd - 3, nd - 2, nd - 4, nd - 1).contiguous()
+    return v.reshape(*lead, N, K)
 
 
 def dequant_matmul(xq: torch.Tensor, wq: torch.Tensor, x_scale: torch.Tensor,

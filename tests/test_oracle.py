@@ -312,3 +312,20 @@ def test_fused_producers_reduce_to_their_parts():
     sc2[:, 2] = 4.0
     qg2, sg2 = O.gather_scale_quant_dense_tokens(x, perm, torch.full((7,), 2), sc2)
     assert torch.equal(qg2.view(torch.uint8), qg.view(torch.uint8)) and torch.equal(sg2, sg * 4.0)
+
+
+def test_preshuffle_layout_by_brute_force():
+    """Element (n, k) must land at flat position ((n // 16) * (K // 64) + k // 64) * 1024 + ((k % 64) // 16) * 256 + (n % 16) * 16 + k % 16."""
+    for lead, N, K in [((), 16, 64), ((), 48, 192), ((3,), 32, 128)]:
+        count = N * K * (lead[0] if lead else 1)
+        src = torch.arange(count, dtype=torch.int32).reshape(*lead, N, K)
+        out = O.preshuffle_b(src)
+        flat_src = src.reshape(-1, N, K)
+        flat_out = out.reshape(-1, N * K)
+        for gi in range(flat_src.shape[0]):
+            for n in range(N):
+                for k in range(0, K, 7):   # every 7th column keeps the loop short and still hits all residues
+                    pos = ((n // 16) * (K // 64) + k // 64) * 1024 + ((k % 64) // 16) * 256 + (n % 16) * 16 + k % 16
+                    assert flat_out[gi, pos] == flat_src[gi, n, k]
+    # it is a permutation: sorting recovers the input
+    assert torch.equal(out.reshape(-1).sort().values, src.reshape(-1))
