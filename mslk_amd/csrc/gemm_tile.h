@@ -15,7 +15,8 @@
 //     (16 consecutive rows, same logical chunk) touch 16 different 16-byte bank groups.  The DMA
 //     cannot scatter inside a wave, so the permutation is applied on the GLOBAL side: lane l of a
 //     load fetches logical chunk (l & 7) ^ swz(row) of its row.
-//   * Two LDS stages; the loads of step k+1 are in flight while step k is multiplied.
+//   * Two XQ buffers and three WQ buffers: while step k is multiplied, the XQ tile of step k+1 and the
+//     WQ tiles of steps k+1 and k+2 are in flight (the weights are the cold, read-once stream).
 // Math
 //   * v_mfma_f32_16x16x128_f8f6f4 (both operands e4m3, unit block scales).  WQ rows are the first
 //     operand and XQ rows the second, so a lane ends up holding 4 consecutive n for one m and
@@ -39,8 +40,9 @@ struct TileShape {
   static constexpr int FN = BN / WAVES_N / 16;  // 16-row n fragments per wave
   static constexpr int A_BYTES = BM * kBK;
   static constexpr int B_BYTES = BN * kBK;
-  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
-  static constexpr int LDS_BYTES = 2 * STAGE_BYTES;
+  static constexpr int A_STAGES = 2;            // XQ tiles: the one being read and the one in flight
+  static constexpr int B_STAGES = 3;            // WQ tiles: one being read, two in flight
+  static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
   static constexpr int LA = BM / 8 / NW;        // wave-level loads of the A tile per wave per step
   static constexpr int LB = BN / 8 / NW;
 };
@@ -111,31 +113,32 @@ struct GemmTile {
   MSLK_AMD_DEVINL static int wave_id() { return __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); }
 
   // DMA load number i (0 .. LA-1 for the XQ tile, 0 .. LB-1 for the WQ tile) of the K step at byte k0.
-  MSLK_AMD_DEVINL void issue_a(char* stage, int k0, int i) {
-    dma16(a_base + k0 + a_off[i], stage + (wave_id() * TS::LA + i) * 1024);
+  // `abuf` / `bbuf` are the LDS buffers that receive the XQ / WQ tile of the K step at byte k0.
+  MSLK_AMD_DEVINL void issue_a(char* abuf, int k0, int i) {
+    dma16(a_base + k0 + a_off[i], abuf + (wave_id() * TS::LA + i) * 1024);
   }
-  MSLK_AMD_DEVINL void issue_b(char* stage, int k0, int i) {
+  MSLK_AMD_DEVINL void issue_b(char* bbuf, int k0, int i) {
     // pre-shuffled: the K step at byte k0 starts 16 rows x k0 bytes into the row group
-    dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], stage + TS::A_BYTES + (wave_id() * TS::LB + i) * 1024);
+    dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
   }
-
-  // All DMA loads of a full K step (128 valid bytes per row) starting at byte k0 into `stage`.
-  MSLK_AMD_DEVINL void issue_loads(char* stage, int k0) {
+  MSLK_AMD_DEVINL void issue_a_all(char* abuf, int k0) {
 #pragma unroll
-    for (int i = 0; i < TS::LA; ++i) issue_a(stage, k0, i);
+    for (int i = 0; i < TS::LA; ++i) issue_a(abuf, k0, i);
+  }
+  MSLK_AMD_DEVINL void issue_b_all(char* bbuf, int k0) {
 #pragma unroll
-    for (int i = 0; i < TS::LB; ++i) issue_b(stage, k0, i);
+    for (int i = 0; i < TS::LB; ++i) issue_b(bbuf, k0, i);
   }
 
   // K tail (K % 128 != 0, K % 16 == 0): only `k_valid` bytes of each row remain.  Chunks at or
   // beyond K are zero-filled with a plain LDS store by the lane that would have fetched them.
-  MSLK_AMD_DEVINL void issue_loads_tail(char* stage, int k0, int k_valid) {
+  MSLK_AMD_DEVINL void issue_loads_tail(char* abuf, char* bbuf, int k0, int k_valid) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
     for (int i = 0; i < TS::LA; ++i) {
       const int row = (wave * TS::LA + i) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swz(row);
-      char* dst = stage + (wave * TS::LA + i) * 1024;
+      char* dst = abuf + (wave * TS::LA + i) * 1024;
       if (chunk * 16 < k_valid) dma16(a_base + k0 + a_off[i], dst);
       else *reinterpret_cast<uint4*>(dst + lane * 16) = make_uint4(0, 0, 0, 0);
     }
@@ -143,7 +146,7 @@ struct GemmTile {
     for (int i = 0; i < TS::LB; ++i) {
       const int row = (wave * TS::LB + i) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swz(row);
-      char* dst = stage + TS::A_BYTES + (wave * TS::LB + i) * 1024;
+      char* dst = bbuf + (wave * TS::LB + i) * 1024;
       const bool valid = PS ? ((wave * TS::LB + i) & 1) * 64 < k_valid : chunk * 16 < k_valid;
       if (valid) dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], dst);
       else *reinterpret_cast<uint4*>(dst + lane * 16) = make_uint4(0, 0, 0, 0);
@@ -177,58 +180,77 @@ struct GemmTile {
       return load_frag(tile, t, fo);
     }
   }
-  MSLK_AMD_DEVINL static const char* a_tile_of(const char* stage) {
-    return stage + (wave_id() / TS::WN) * (TS::kBM / TS::WM) * kBK;
+  // The part of an XQ / WQ buffer this wave multiplies.
+  MSLK_AMD_DEVINL static const char* a_tile_of(const char* abuf) {
+    return abuf + (wave_id() / TS::WN) * (TS::kBM / TS::WM) * kBK;
   }
-  MSLK_AMD_DEVINL static const char* b_tile_of(const char* stage) {
-    return stage + TS::A_BYTES + (wave_id() % TS::WN) * (TS::kBN / TS::WN) * kBK;
+  MSLK_AMD_DEVINL static const char* b_tile_of(const char* bbuf) {
+    return bbuf + (wave_id() % TS::WN) * (TS::kBN / TS::WN) * kBK;
   }
   // First fragments of a K step: all XQ fragments and WQ fragment 0.
-  MSLK_AMD_DEVINL void load_first_frags(const char* stage, v8i (&xf)[TS::FM], v8i& wf0) {
+  MSLK_AMD_DEVINL void load_first_frags(const char* abuf, const char* bbuf, v8i (&xf)[TS::FM], v8i& wf0) {
     const FragOff fo = frag_off();
-    wf0 = load_frag_b(b_tile_of(stage), 0, fo);
+    wf0 = load_frag_b(b_tile_of(bbuf), 0, fo);
 #pragma unroll
-    for (int tm = 0; tm < TS::FM; ++tm) xf[tm] = load_frag(a_tile_of(stage), tm, fo);
+    for (int tm = 0; tm < TS::FM; ++tm) xf[tm] = load_frag(a_tile_of(abuf), tm, fo);
   }
 
-  // One K step of MFMAs out of stage `cur`; xf / wf0 (its XQ fragments and WQ fragment 0) are
-  // already in registers.  The step is software-pipelined across the workgroup barrier:
-  //   * DMA: the global -> LDS loads of the FOLLOWING K step (byte offset k_next, stage `nxt`) are issued
-  //     between the MFMA groups of the first half of the step, so that their issue cost hides under
-  //     matrix work and they have half a step to land;
-  //   * NEXT: before the last MFMA group the wave waits for its DMA and all its LDS reads and passes the
-  //     barrier (after which stage `nxt` is complete and nobody reads `cur` any more).  The operands of
-  //     the last group are in registers; each XQ fragment is re-loaded from `nxt` right after the MFMA
-  //     that used it last, so the barrier and the LDS latency overlap with matrix work and the
-  //     following step starts with its first fragments already on their way.
-  template <bool DMA, bool NEXT>
-  MSLK_AMD_DEVINL void step(const char* cur, char* nxt, int k_next, v4f (&acc)[TS::FN][TS::FM],
-                            v8i (&xf)[TS::FM], v8i& wf0) {
+  // Waits until at most `pending` of this wave's DMA loads (the youngest ones) are still in flight and
+  // all its LDS reads have returned, then passes the workgroup barrier.
+  template <int PENDING>
+  MSLK_AMD_DEVINL static void wait_and_barrier() {
+    static_assert(PENDING >= 0 && PENDING < 16, "vmcnt immediate");
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");                  // no LDS access moves across the barrier at compile time
+    __builtin_amdgcn_s_waitcnt(0x0070 | PENDING);   // vmcnt(PENDING) lgkmcnt(0), expcnt untouched
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // One K step of MFMAs on the WQ tile in `b_cur`; xf / wf0 (the step's XQ fragments and WQ fragment 0)
+  // are already in registers.  The step is software-pipelined across the workgroup barrier and the
+  // weight stream runs two steps ahead:
+  //   * DMA_A / DMA_B: the global -> LDS loads of the XQ tile of the NEXT step (byte offset k_a, buffer
+  //     `a_nxt`) and of the WQ tile of the step AFTER it (byte offset k_b, buffer `b_far`) are issued
+  //     between the MFMA groups of the first half of the step, XQ first, so that their issue cost hides
+  //     under matrix work.  Weights are the cold stream (read once from HBM); giving them two steps to
+  //     land keeps twice as many bytes in flight per CU as a plain double buffer.
+  //   * NEXT: before the last MFMA group the wave waits for everything but the WQ loads it issued in this
+  //     step, and for all its LDS reads, and passes the barrier (after which `a_nxt` and `b_nxt` are
+  //     complete and nobody reads `b_cur` any more).  The operands of the last group are in registers;
+  //     each XQ fragment is re-loaded from `a_nxt` right after the MFMA that used it last, so the barrier
+  //     and the LDS latency overlap with matrix work and the following step starts with its first
+  //     fragments already on their way.
+  template <bool DMA_A, bool DMA_B, bool NEXT>
+  MSLK_AMD_DEVINL void step(const char* b_cur, char* a_nxt, const char* b_nxt, char* b_far, int k_a, int k_b,
+                            v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
     constexpr int HALF = TS::FN / 2;
-    static_assert(TS::LA % HALF == 0 && TS::LB % HALF == 0, "DMA loads spread evenly over the first half");
-    constexpr int PA = TS::LA / HALF, PB = TS::LB / HALF;
+    static_assert((TS::LA + TS::LB) % HALF == 0, "DMA loads spread evenly over the first half");
+    constexpr int NDMA = (TS::LA + TS::LB) / HALF;   // DMA loads per MFMA group
+    static_assert(NDMA <= TS::FM, "one DMA per MFMA slot");
     const FragOff fo = frag_off();
-    const char* b_tile = b_tile_of(cur);
+    const char* b_tile = b_tile_of(b_cur);
     v8i wf = wf0;
 #pragma unroll
     for (int tn = 0; tn < TS::FN - 1; ++tn) {
       // Issue order inside a group: the read of the next WQ fragment follows the first MFMA, the DMA
       // loads follow the last MFMAs, one each.  Every DMA sits in the shadow of an MFMA, and the
       // LDS reads issued before it are at least four MFMAs old: the compiler orders all earlier LDS
-      // reads before a DMA write (it cannot see that the two stages are disjoint), so a DMA right
+      // reads before a DMA write (it cannot see that the buffers are disjoint), so a DMA right
       // behind a fresh read would stall on that read's latency.
-      constexpr int NDMA = PA + PB;
-      static_assert(NDMA <= TS::FM, "one DMA per MFMA slot");
       v8i wf_next;
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) {
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
         if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
-        if constexpr (DMA) {
-          const int d = tm - (TS::FM - NDMA);
-          if (tn < HALF && d >= 0) {
-            if (d < PA) issue_a(nxt, k_next, tn * PA + d);
-            else issue_b(nxt, k_next, tn * PB + (d - PA));
+        const int d = tm - (TS::FM - NDMA);
+        if (tn < HALF && d >= 0) {
+          const int q = tn * NDMA + d;   // all XQ loads are older than all WQ loads of the step
+          if (q < TS::LA) {
+            if constexpr (DMA_A) issue_a(a_nxt, k_a, q);
+          } else {
+            if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -237,10 +259,10 @@ struct GemmTile {
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (NEXT) {
-      __syncthreads();  // s_waitcnt vmcnt(0) lgkmcnt(0); s_barrier
-      wf0 = load_frag_b(b_tile_of(nxt), 0, fo);
+      wait_and_barrier<DMA_B ? TS::LB : 0>();
+      wf0 = load_frag_b(b_tile_of(b_nxt), 0, fo);
     }
-    const char* a_next = a_tile_of(nxt);
+    const char* a_next = a_tile_of(a_nxt);
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
       acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
@@ -270,28 +292,43 @@ struct GemmTile {
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    char* cur = lds;
-    char* nxt = lds + TS::STAGE_BYTES;
+    char* a_cur = lds;
+    char* a_nxt = lds + TS::A_BYTES;
+    char* b_cur = lds + 2 * TS::A_BYTES;
+    char* b_nxt = b_cur + TS::B_BYTES;
+    char* b_far = b_nxt + TS::B_BYTES;
     const int KT = K / kBK;           // full steps
     const int k_tail = K - KT * kBK;  // 0 or a multiple of 16
     v8i xf[TS::FM], wf0;
     if (KT > 0) {
-      issue_loads(cur, 0);
-      __syncthreads();
-      load_first_frags(cur, xf, wf0);
-      for (int kt = 0; kt < KT - 1; ++kt) {
-        step<true, true>(cur, nxt, (kt + 1) * kBK, acc, xf, wf0);
-        char* t = cur; cur = nxt; nxt = t;
+      issue_a_all(a_cur, 0);
+      issue_b_all(b_cur, 0);
+      if (KT > 1) {
+        issue_b_all(b_nxt, kBK);
+        wait_and_barrier<TS::LB>();
+      } else {
+        wait_and_barrier<0>();
       }
-      step<false, false>(cur, nxt, 0, acc, xf, wf0);
-      { char* t = cur; cur = nxt; nxt = t; }
+      load_first_frags(a_cur, b_cur, xf, wf0);
+      // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
+      for (int kt = 0; kt < KT - 2; ++kt) {
+        step<true, true, true>(b_cur, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
+        { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
+        { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
+      }
+      if (KT > 1) {
+        step<true, false, true>(b_cur, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
+        { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
+        { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
+      }
+      step<false, false, false>(b_cur, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
     }
     if (k_tail > 0) {
-      __syncthreads();   // everybody is done reading `cur` (consumed two steps ago) before it is refilled
-      issue_loads_tail(cur, KT * kBK, k_tail);
+      __syncthreads();   // everybody is done with the buffers of the full steps before one pair is refilled
+      issue_loads_tail(a_nxt, b_nxt, KT * kBK, k_tail);
       __syncthreads();
-      load_first_frags(cur, xf, wf0);
-      step<false, false>(cur, nxt, 0, acc, xf, wf0);
+      load_first_frags(a_nxt, b_nxt, xf, wf0);
+      step<false, false, false>(b_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
     }
     __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
