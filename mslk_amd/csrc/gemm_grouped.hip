@@ -37,8 +37,10 @@ __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
   const int per_xcd = (tab.total_tiles + kXcds - 1) / kXcds;
   const int t = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
   if (t >= tab.total_tiles) return;
-  int gi = 0;
-  while (gi + 1 < tab.count && t >= tab.g[gi + 1].tile_begin) ++gi;
+  // group lookup in one step: lane i compares against the first tile of group i (count <= 64, begins ascend)
+  const int lane = threadIdx.x & 63;
+  const int begin = lane < tab.count ? tab.g[lane].tile_begin : 0x7FFFFFFF;
+  const int gi = __builtin_amdgcn_readfirstlane(__popcll(__ballot(t >= begin)) - 1);
   const GroupDesc& d = tab.g[gi];
   const int tiles_m = (d.M + BM - 1) / BM, tiles_n = (d.N + BN - 1) / BN;
   int tm, tn;
@@ -66,6 +68,11 @@ struct GroupSpan {
   int t;         // tile index inside the group
 };
 
+MSLK_AMD_DEVINL int64_t uniform64(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v), hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 template <int LAYOUT, int BM, int BN>
 MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
@@ -91,25 +98,57 @@ MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
       return b >= 0 && e >= b && e <= p.K;
     }
   } else {
+    // The G extents are read 64 at a time, one per lane, and turned into tile ranges by a wave-level
+    // prefix sum, so the lookup costs one memory round trip instead of G dependent ones.
     const int fixed_tiles = LAYOUT == kGroupsOffsetsN ? tiles_m : tiles_n;
     const int blk = LAYOUT == kGroupsOffsetsN ? BN : BM;
     const int64_t total = LAYOUT == kGroupsOffsetsN ? p.N : p.M;
-    int64_t b = 0;
-    for (int gi = 0; gi < p.G; ++gi) {
-      int64_t len;
+    const int lane = threadIdx.x & 63;
+    int64_t carry_tiles = 0, carry_len = 0;
+    for (int base = 0; base < p.G; base += 64) {
+      const int gi = base + lane;
+      const bool in = gi < p.G;
+      int64_t start = 0, len = 0;
       if constexpr (LAYOUT == kGroupsSizesM) {
-        len = static_cast<const int64_t*>(p.layout)[gi];
+        if (in) len = static_cast<const int64_t*>(p.layout)[gi];
+        int64_t incl_len = len;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const int64_t v = __shfl_up(incl_len, d, 64);
+          if (lane >= d) incl_len += v;
+        }
+        start = carry_len + incl_len - len;
+        carry_len += __shfl(incl_len, 63, 64);
       } else {
-        len = (int64_t) static_cast<const int32_t*>(p.layout)[gi] - b;
+        const int32_t* off = static_cast<const int32_t*>(p.layout);
+        if (in) {
+          start = gi ? off[gi - 1] : 0;
+          len = (int64_t)off[gi] - start;
+        }
       }
-      if (len < 0 || b + len > total) return false;   // inconsistent group data: touch nothing
-      const int64_t tiles = ((len + blk - 1) / blk) * fixed_tiles;
-      if (t < tiles) {
-        sp.gi = gi; sp.o0 = b; sp.len = (int)len; sp.t = t;
+      const bool bad = in && (len < 0 || start < 0 || start + len > total);   // inconsistent group data
+      const int64_t tiles = (in && !bad) ? ((len + blk - 1) / blk) * fixed_tiles : 0;
+      int64_t incl = tiles;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int64_t v = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += v;
+      }
+      const int64_t excl = carry_tiles + incl - tiles;
+      const bool hit = tiles > 0 && t >= excl && t < excl + tiles;
+      const unsigned long long hit_mask = __ballot(hit), bad_mask = __ballot(bad);
+      if (hit_mask != 0) {
+        const int src = __ffsll((long long)hit_mask) - 1;
+        if (bad_mask & ((1ull << src) - 1ull)) return false;   // a group before this one is inconsistent: touch nothing
+        // the results are the same in every lane: say so, so that the tile's addresses live in scalar registers
+        sp.gi = base + src;
+        sp.o0 = uniform64(__shfl(start, src, 64));
+        sp.len = __builtin_amdgcn_readfirstlane((int)__shfl(len, src, 64));
+        sp.t = t - __builtin_amdgcn_readfirstlane((int)__shfl(excl, src, 64));
         return true;
       }
-      t -= (int)tiles;
-      b += len;
+      if (bad_mask != 0) return false;
+      carry_tiles += __shfl(incl, 63, 64);
     }
     return false;
   }
