@@ -197,3 +197,51 @@ def test_argument_checks_follow_the_reference():
     e = torch.ops.mslk.f8f8bf16_rowwise_grouped_mm(XQ[:0], WQ, xs[:0], ws, torch.zeros(2, dtype=torch.int32, device=DEV),
                                                    torch.empty(0, 512, dtype=torch.bfloat16, device=DEV))
     assert e.shape == (0, 512)
+
+
+def test_graph_replay_follows_device_side_group_sizes():
+    """The group extents are read on the device, so a captured graph must follow offsets / sizes that
+    change between replays (test/gemm/gemm_test.py:652,776 capture these ops); every replay is compared
+    with an eager call on the same extents, with eager work between the replays."""
+    g = torch.Generator().manual_seed(41)
+    G, N, K, total = 4, 512, 512, 700
+    xq, xs = _quant(total, K, g)
+    wq, ws = _quant(G * N, K, g, 0.02)
+    XQ, WQ, XS, WS = xq.to(DEV), wq.view(G, N, K).to(DEV), xs.to(DEV), ws.view(G, N).to(DEV)
+    ends = torch.zeros(G, dtype=torch.int32, device=DEV)
+    sizes = torch.zeros(G, dtype=torch.int64, device=DEV)
+    out = _sentinel(total, N)
+    splits = [[100, 200, 300, 100], [0, 700, 0, 0], [1, 2, 3, 4], [175, 175, 175, 175]]
+
+    def set_split(ms):
+        ends.copy_(torch.tensor(ms, dtype=torch.int64).cumsum(0).to(torch.int32))
+        sizes.copy_(torch.tensor(ms, dtype=torch.int64))
+
+    set_split(splits[0])
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):   # warm-up outside capture
+        torch.ops.mslk.f8f8bf16_rowwise_grouped_mm(XQ, WQ, XS, WS, ends, out)
+        torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked(XQ, WQ, XS, WS, sizes)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        torch.ops.mslk.f8f8bf16_rowwise_grouped_mm(XQ, WQ, XS, WS, ends, out)
+        y_stacked = torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked(XQ, WQ, XS, WS, sizes)
+    for ms in splits:
+        set_split(ms)
+        out.fill_(SENTINEL)
+        y_stacked.fill_(SENTINEL)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = torch.ops.mslk.f8f8bf16_rowwise_grouped_mm(XQ, WQ, XS, WS, ends, _sentinel(total, N))   # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager) and torch.equal(y_stacked, eager)
+        r0 = 0
+        for gi, m in enumerate(ms):
+            if m:
+                assert_gemm_close(out[r0:r0 + m], O.dequant_matmul(xq[r0:r0 + m], wq[gi * N:(gi + 1) * N], xs[r0:r0 + m],
+                                                                   ws[gi * N:(gi + 1) * N]), f"split {ms} group {gi}")
+            r0 += m
+        assert (out[r0:] == SENTINEL).all()
