@@ -287,3 +287,23 @@ def test_fp16_output_matches_oracle(M, N, K):
     assert ((yf - ybf).abs()[normal] <= yf.abs()[normal] * (2.0 ** -8 + 2.0 ** -11) * 1.0001).all()
     differs = (yf.bfloat16() != yb).float().mean().item()
     assert differs < 0.09
+
+
+def test_seeded_random_shape_sweep():
+    """Sixty seeded shapes across the dispatch boundaries (skinny <-> tiled at M = 64, 128^2 <-> 256^2 tiles,
+    K tails, K % 16 != 0 -> generic kernel, N not a multiple of 8), with and without bias, both output types."""
+    g = torch.Generator().manual_seed(2024)
+    for case in range(60):
+        M = int(torch.randint(1, 400, (1,), generator=g))
+        N = int(torch.randint(1, 700, (1,), generator=g))
+        K = int(torch.randint(1, 80, (1,), generator=g)) * (16 if case % 5 else 1)
+        if case % 7 == 0:
+            M, N = M * 9, N * 5          # enough tiles for the 256 x 256 shape
+        xq, wq, xs, ws = _random_problem(M, N, K, g)
+        bias = (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16 if case % 2 else torch.float32) if case % 3 == 0 else None
+        op = torch.ops.mslk.f8f8f16_rowwise if case % 4 == 1 else torch.ops.mslk.f8f8bf16_rowwise
+        y = op(*_gpu(xq, wq, xs, ws), bias=None if bias is None else bias.to(DEV))
+        torch.cuda.synchronize()
+        ref = O.dequant_matmul(xq, wq, xs, ws, None if bias is None else bias.float())
+        assert y.shape == (M, N)
+        assert_gemm_close(y, ref, f"case {case}: {M}x{N}x{K} bias={None if bias is None else bias.dtype} op={op}")
