@@ -68,6 +68,21 @@ int mslk_amd_quantize_fp8_row_jagged(const void* x, int x_dtype, int64_t rows, i
                                      void* stream);
 
 /*
+ * The quantizer with the arithmetic of the reference's GPU (Triton) branch instead of its torch branch
+ * (reference: _kernel_quantize_fp8_row, mslk/quantize/triton/fp8_quantize.py:131-207; eps default 1/512,
+ * same file 215,246-247):
+ *   amax = clamp(max|x|, eps [, *scale_ub]);  scale = fl32(amax / 448);
+ *   code = e4m3fn_rne(clamp(fl32(fl32(x) / scale), -448, 448))      (IEEE divisions, saturating)
+ * Arguments as mslk_amd_quantize_fp8_row_jagged; zero_start_index may be NULL (then index_dtype and
+ * rows_per_group are ignored).  The bits differ from mslk_amd_quantize_fp8_row in the last place of some
+ * scales and codes, in the lower bound of amax, and in saturating where scale_ub cuts the maximum.
+ */
+int mslk_amd_quantize_fp8_row_triton_arithmetic(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t x_row_stride,
+                                                void* xq, int64_t K_out, float* scale, const float* scale_ub, float eps,
+                                                const void* zero_start_index, int index_dtype, int64_t rows_per_group,
+                                                void* stream);
+
+/*
  * Row-wise dequantization to bf16.  Replaces dequantize_fp8_row
  * (reference: mslk/quantize/triton/fp8_quantize.py:1060-1113 kernel, 1140-1182 wrapper):
  *   out[r, k] = bf16_rne( fl32( f32(xq[r, k]) * scale[r] ) )

@@ -22,6 +22,8 @@ SIGNATURES = {
                                           c_void_p, c_void_p, c_void_p]),
     "mslk_amd_quantize_fp8_row_jagged": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64,
                                                  c_void_p, c_void_p, c_void_p, c_int, c_int64, c_void_p]),
+    "mslk_amd_quantize_fp8_row_triton_arithmetic": (c_int, [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_int64,
+                                                            c_void_p, c_void_p, c_float, c_void_p, c_int, c_int64, c_void_p]),
     "mslk_amd_silu_mul_quant": (c_int, [c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p,
                                         c_void_p, c_void_p, c_int, c_void_p]),
     "mslk_amd_gather_scale_quant_dense_tokens": (c_int, [c_void_p, c_int, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int,

@@ -45,7 +45,7 @@ int mslk_amd_quantize_fp8_row(const void* x, int x_dtype, int64_t rows, int64_t 
   if (rows > kIntMax) return fail("quantize_fp8_row: rows (%lld) exceeds 2^31-1", (long long)rows);
   if (!x || !xq || !scale) return fail("quantize_fp8_row: null pointer");
   return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub, nullptr, 0, 1,
-                                           (hipStream_t)stream),
+                                           0, 0.f, (hipStream_t)stream),
                    "quantize_fp8_row launch");
 }
 
@@ -66,8 +66,30 @@ int mslk_amd_quantize_fp8_row_jagged(const void* x, int x_dtype, int64_t rows, i
   if (!x || !xq || !scale || !zero_start_index) return fail("quantize_fp8_row_jagged: null pointer");
   return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub,
                                            zero_start_index, index_dtype == MSLK_AMD_INDEX_I32, rows_per_group,
-                                           (hipStream_t)stream),
+                                           0, 0.f, (hipStream_t)stream),
                    "quantize_fp8_row_jagged launch");
+}
+
+int mslk_amd_quantize_fp8_row_triton_arithmetic(const void* x, int x_dtype, int64_t rows, int64_t K, int64_t x_row_stride,
+                                                void* xq, int64_t K_out, float* scale, const float* scale_ub, float eps,
+                                                const void* zero_start_index, int index_dtype, int64_t rows_per_group,
+                                                void* stream) {
+  const char* op = "quantize_fp8_row_triton_arithmetic";
+  if (x_dtype < 0 || x_dtype > 2) return fail("%s: unsupported input dtype code %d", op, x_dtype);
+  if (rows < 0 || K <= 0) return fail("%s: rows must be >= 0 and K > 0 (got %lld, %lld)", op, (long long)rows, (long long)K);
+  if (K_out < K) return fail("%s: K_out (%lld) < K (%lld)", op, (long long)K_out, (long long)K);
+  if (!(eps > 0.f)) return fail("%s: eps must be positive", op);
+  if (zero_start_index != nullptr) {
+    if (index_dtype != MSLK_AMD_INDEX_I64 && index_dtype != MSLK_AMD_INDEX_I32) return fail("%s: unsupported index dtype code %d", op, index_dtype);
+    if (rows_per_group <= 0 || rows % rows_per_group != 0)
+      return fail("%s: rows (%lld) must be a multiple of rows_per_group (%lld)", op, (long long)rows, (long long)rows_per_group);
+  }
+  if (rows == 0) return 0;
+  if (rows > kIntMax) return fail("%s: rows (%lld) exceeds 2^31-1", op, (long long)rows);
+  if (!x || !xq || !scale) return fail("%s: null pointer", op);
+  return check_hip(launch_quantize_fp8_row(x, x_dtype, rows, K, x_row_stride, xq, K_out, scale, scale_ub, zero_start_index,
+                                           index_dtype == MSLK_AMD_INDEX_I32, rows_per_group, 1, eps, (hipStream_t)stream),
+                   "quantize_fp8_row_triton_arithmetic launch");
 }
 
 int mslk_amd_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out, void* stream) {

@@ -10,7 +10,7 @@ namespace mslk_amd {
 hipError_t launch_quantize_fp8_row(const void* x, int dtype, int64_t rows, int64_t K, int64_t in_stride,
                                    void* xq, int64_t K_out, float* scale, const float* scale_ub,
                                    const void* zero_start, int zero_start_is_i32, int64_t rows_per_group,
-                                   hipStream_t s);
+                                   int triton_arithmetic, float triton_eps, hipStream_t s);
 hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t rows, int64_t K, void* out,
                                      hipStream_t s);
 // WQ [G, N, K] row-major -> the blocked layout the *_preshuffle GEMMs read (N % 16 == 0, K % 64 == 0).

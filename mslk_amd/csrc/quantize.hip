@@ -8,6 +8,11 @@
 //   code  = e4m3fn_rne(fl32(fl32(x) * inv))            (no saturation: > 464 becomes NaN)
 //   scale = fl32(1 / inv)
 //
+// TRITON = true selects the arithmetic of the reference's GPU (Triton) kernel instead
+// (mslk/quantize/triton/fp8_quantize.py:131-207): amax clamped at `eps` (default 1/512) [and *scale_ub],
+//   scale = fl32(amax / 448);  code = e4m3fn_rne(clamp(fl32(fl32(x) / scale), -448, 448))
+// with IEEE-correct divisions (div_rn) and saturation.
+//
 // The pass is HBM-bound (2 B in + 1 B out per element for bf16), so the kernel is organised
 // around 128-bit coalesced loads that stay in registers between the amax pass and the convert
 // pass: a row is owned by a "team" of 64 lanes (one wavefront) or 256 lanes (one workgroup);
@@ -96,8 +101,9 @@ MSLK_AMD_DEVINL uint32_t finish_absmax_bits(uint32_t m) {
   return max(m & 0xFFFFu, m >> 16);
 }
 
-template <int DTYPE>
-MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float inv) {
+// `factor` is the multiplier `inv` of the torch-branch formula, or the divisor `scale` of the Triton one.
+template <int DTYPE, bool TRITON>
+MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float factor) {
   float f[8];
   if constexpr (DTYPE == 2) {
     const uint32_t w[8] = {v.lo.x, v.lo.y, v.lo.z, v.lo.w, v.hi.x, v.hi.y, v.hi.z, v.hi.w};
@@ -112,7 +118,10 @@ MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float inv) {
     }
   }
 #pragma unroll
-  for (int i = 0; i < 8; ++i) f[i] = f[i] * inv;
+  for (int i = 0; i < 8; ++i) {
+    if constexpr (TRITON) f[i] = __builtin_fminf(__builtin_fmaxf(f[i] / factor, -448.0f), 448.0f);
+    else f[i] = f[i] * factor;
+  }
   uint2 r;
   r.x = cvt_pk_e4m3fn(f[0], f[1]) | (cvt_pk_e4m3fn(f[2], f[3]) << 16);
   r.y = cvt_pk_e4m3fn(f[4], f[5]) | (cvt_pk_e4m3fn(f[6], f[7]) << 16);
@@ -120,8 +129,16 @@ MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float inv) {
 }
 
 // amax (as fp32, NaN if the row holds a NaN) -> (inv, scale) of the reference formula.
-template <int DTYPE>
-MSLK_AMD_DEVINL void scales_from_amax(float amax, const float* scale_ub, float& inv, float& scale) {
+template <int DTYPE, bool TRITON>
+MSLK_AMD_DEVINL void scales_from_amax(float amax, const float* scale_ub, float triton_eps, float& inv, float& scale) {
+  if constexpr (TRITON) {
+    // tl.maximum / tl.clamp against fp32 constants, then div_rn(cur_max, MAX_FP8); `inv` carries the divisor
+    float c = (amax < triton_eps) ? triton_eps : amax;
+    if (scale_ub != nullptr) c = (c > *scale_ub) ? *scale_ub : c;
+    scale = c / 448.0f;
+    inv = scale;
+    return;
+  }
   const float eps = Traits<DTYPE>::eps();
   float c = (amax < eps) ? eps : amax;  // comparisons are false for NaN: NaN propagates
   if (scale_ub != nullptr) {
@@ -141,6 +158,7 @@ struct JaggedRows {
   const void* zero_start;   // nullptr: every row is live
   int64_t rows_per_group;
   int index_is_i32;
+  float triton_eps;         // lower bound of amax in the TRITON arithmetic
 };
 
 MSLK_AMD_DEVINL bool row_is_live(const JaggedRows& j, int64_t row) {
@@ -169,7 +187,7 @@ MSLK_AMD_DEVINL uint32_t team_max(uint32_t m, uint32_t* smem, int team_in_block)
 }
 
 // Vector path: K % 8 == 0, row starts 16-byte aligned, output rows 8-byte aligned.
-template <int DTYPE, int TEAM, int NV, bool CACHED>
+template <int DTYPE, int TEAM, int NV, bool CACHED, bool TRITON>
 __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
     const void* __restrict__ x, int64_t rows, int K, int64_t in_stride, uint8_t* __restrict__ out,
     int64_t out_stride, float* __restrict__ scale, const float* __restrict__ scale_ub, JaggedRows jag) {
@@ -203,7 +221,7 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
   if (!valid) return;
 
   float inv, sc;
-  scales_from_amax<DTYPE>(Traits<DTYPE>::abs_bits_to_f32(m), scale_ub, inv, sc);
+  scales_from_amax<DTYPE, TRITON>(Traits<DTYPE>::abs_bits_to_f32(m), scale_ub, jag.triton_eps, inv, sc);
   if (lane == 0) scale[row] = sc;
 
   uint2* out_row = reinterpret_cast<uint2*>(out + row * out_stride);
@@ -213,18 +231,18 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = i * TEAM + lane;
-      if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE>(cache[i], inv));
+      if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(cache[i], inv));
     }
   } else {
     for (int idx = lane; idx < nvec; idx += TEAM)
-      store8_stream(out_row + idx, quantize_vec8<DTYPE>(load_vec8<DTYPE>(row_ptr, idx), inv));
+      store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(load_vec8<DTYPE>(row_ptr, idx), inv));
   }
   // zero padding columns [K, out_stride)
   for (int64_t k = K + lane; k < out_stride; k += TEAM) out[row * out_stride + k] = 0;
 }
 
 // Generic path: any K, any alignment; one workgroup per row, scalar accesses, two passes.
-template <int DTYPE>
+template <int DTYPE, bool TRITON>
 __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
     const void* __restrict__ x, int64_t rows, int64_t K, int64_t in_stride, uint8_t* __restrict__ out,
     int64_t out_stride, float* __restrict__ scale, const float* __restrict__ scale_ub, JaggedRows jag) {
@@ -240,7 +258,7 @@ __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
   }
   m = team_max<256>(m, smem, 0);
   float inv, sc;
-  scales_from_amax<DTYPE>(Traits<DTYPE>::abs_bits_to_f32(m), scale_ub, inv, sc);
+  scales_from_amax<DTYPE, TRITON>(Traits<DTYPE>::abs_bits_to_f32(m), scale_ub, jag.triton_eps, inv, sc);
   if (threadIdx.x == 0) scale[row] = sc;
   for (int64_t k = threadIdx.x; k < out_stride; k += 256) {
     uint8_t code = 0;
@@ -248,7 +266,9 @@ __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
       float f;
       if constexpr (DTYPE == 2) f = xr[k];
       else f = Traits<DTYPE>::to_f32(xr[k]);
-      code = (uint8_t)(cvt_pk_e4m3fn(f * inv, 0.0f) & 0xFFu);
+      if constexpr (TRITON) f = __builtin_fminf(__builtin_fmaxf(f / inv, -448.0f), 448.0f);
+      else f = f * inv;
+      code = (uint8_t)(cvt_pk_e4m3fn(f, 0.0f) & 0xFFu);
     }
     out[row * out_stride + k] = code;
   }
@@ -293,7 +313,7 @@ __global__ void cast_e4m3fn_kernel(const float* __restrict__ in, int64_t n, uint
     out[i] = (uint8_t)(cvt_pk_e4m3fn(in[i], 0.0f) & 0xFFu);
 }
 
-template <int DTYPE>
+template <int DTYPE, bool TRITON>
 hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_stride, uint8_t* out,
                              int64_t out_stride, float* scale, const float* scale_ub, JaggedRows jag,
                              hipStream_t s) {
@@ -303,7 +323,7 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
                       (reinterpret_cast<uintptr_t>(x) % 16 == 0) && (out_stride % 8 == 0) &&
                       (reinterpret_cast<uintptr_t>(out) % 8 == 0);
   if (!vec_ok) {
-    quantize_rows_generic_kernel<DTYPE><<<dim3((unsigned)rows), dim3(256), 0, s>>>(
+    quantize_rows_generic_kernel<DTYPE, TRITON><<<dim3((unsigned)rows), dim3(256), 0, s>>>(
         x, rows, K, in_stride, out, out_stride, scale, scale_ub, jag);
     return hipGetLastError();
   }
@@ -312,17 +332,17 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
   if (K <= kWave * 8 * NV && rows >= 2048) {
     const unsigned blocks = (unsigned)((rows + 3) / 4);
     if (K <= kWave * 8 * 4)
-      quantize_rows_vec_kernel<DTYPE, 64, 4, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+      quantize_rows_vec_kernel<DTYPE, 64, 4, true, TRITON><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
     else if (K <= kWave * 8 * 8)
-      quantize_rows_vec_kernel<DTYPE, 64, 8, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+      quantize_rows_vec_kernel<DTYPE, 64, 8, true, TRITON><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
     else
-      quantize_rows_vec_kernel<DTYPE, 64, NV, true><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+      quantize_rows_vec_kernel<DTYPE, 64, NV, true, TRITON><<<blocks, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else if (K <= 256 * 8 * 4) {
-    quantize_rows_vec_kernel<DTYPE, 256, 4, true><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+    quantize_rows_vec_kernel<DTYPE, 256, 4, true, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else if (K <= 256 * 8 * NV) {
-    quantize_rows_vec_kernel<DTYPE, 256, NV, true><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+    quantize_rows_vec_kernel<DTYPE, 256, NV, true, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else {
-    quantize_rows_vec_kernel<DTYPE, 256, 1, false><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+    quantize_rows_vec_kernel<DTYPE, 256, 1, false, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   }
   return hipGetLastError();
 }
@@ -332,13 +352,20 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
 hipError_t launch_quantize_fp8_row(const void* x, int dtype, int64_t rows, int64_t K, int64_t in_stride,
                                    void* xq, int64_t K_out, float* scale, const float* scale_ub,
                                    const void* zero_start, int zero_start_is_i32, int64_t rows_per_group,
-                                   hipStream_t s) {
+                                   int triton_arithmetic, float triton_eps, hipStream_t s) {
   uint8_t* out = reinterpret_cast<uint8_t*>(xq);
-  const JaggedRows jag{zero_start, rows_per_group > 0 ? rows_per_group : 1, zero_start_is_i32};
+  const JaggedRows jag{zero_start, rows_per_group > 0 ? rows_per_group : 1, zero_start_is_i32, triton_eps};
+  if (triton_arithmetic) {
+    switch (dtype) {
+      case 0: return launch_quantize_t<0, true>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+      case 1: return launch_quantize_t<1, true>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+      default: return launch_quantize_t<2, true>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+    }
+  }
   switch (dtype) {
-    case 0: return launch_quantize_t<0>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
-    case 1: return launch_quantize_t<1>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
-    default: return launch_quantize_t<2>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+    case 0: return launch_quantize_t<0, false>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+    case 1: return launch_quantize_t<1, false>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
+    default: return launch_quantize_t<2, false>(x, rows, K, in_stride, out, K_out, scale, scale_ub, jag, s);
   }
 }
 

@@ -38,7 +38,8 @@ class _on_device:
 
 
 def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, align_rows_to: Optional[int] = None,
-                   zero_start_index_M: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                   zero_start_index_M: Optional[torch.Tensor] = None, triton_eps: Optional[float] = None
+                   ) -> Tuple[torch.Tensor, torch.Tensor]:
     if a.dtype not in _DTYPE_CODE:
         raise RuntimeError(f"quantize_fp8_row: unsupported input dtype {a.dtype} (bf16, fp16, fp32 are supported)")
     if a.dim() < 1:
@@ -69,6 +70,7 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
     if scale_ub is not None:
         scale_ub = scale_ub.to(device=a.device, dtype=torch.float32).reshape(-1)[:1].contiguous()
         ub_ptr = scale_ub.data_ptr()
+    zs_ptr, zs_code, rows_per_group = None, 0, 1
     if zero_start_index_M is not None:
         # One entry per [N, K] matrix of the input viewed as [B, M, N, K] (fp8_quantize.py:236-243).
         rows_per_group = a.shape[-2] if a.dim() >= 2 else 1
@@ -81,12 +83,21 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
             raise RuntimeError(f"zero_start_index_M must have one entry per group of {rows_per_group} rows "
                                f"({rows // max(rows_per_group, 1)} entries), got {zs.numel()}")
         zs = zs.contiguous()
-        if rows > 0:
-            with _on_device(a.device):
-                _lib.check(_lib.lib().mslk_amd_quantize_fp8_row_jagged(
-                    a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
-                    scale.data_ptr(), ub_ptr, zs.data_ptr(), 0 if zs.dtype == torch.int64 else 1, rows_per_group,
-                    _stream_ptr(a.device)))
+        zs_ptr, zs_code = zs.data_ptr(), (0 if zs.dtype == torch.int64 else 1)
+    if rows == 0:
+        return xq, scale
+    if triton_eps is not None:
+        # arithmetic of the reference's Triton kernel (fp8_quantize.py:131-207) instead of its torch branch
+        with _on_device(a.device):
+            _lib.check(_lib.lib().mslk_amd_quantize_fp8_row_triton_arithmetic(
+                a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out, scale.data_ptr(), ub_ptr,
+                float(triton_eps), zs_ptr, zs_code, rows_per_group, _stream_ptr(a.device)))
+        return xq, scale
+    if zs_ptr is not None:
+        with _on_device(a.device):
+            _lib.check(_lib.lib().mslk_amd_quantize_fp8_row_jagged(
+                a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
+                scale.data_ptr(), ub_ptr, zs_ptr, zs_code, rows_per_group, _stream_ptr(a.device)))
         return xq, scale
     if rows > 0:
         with _on_device(a.device):
@@ -96,7 +107,7 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
     return xq, scale
 
 
-def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None, zero_start_index_M=None):
+def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None, zero_start_index_M=None, triton_eps=None):
     # shape function of the reference (fp8_quantize.py:381-407)
     K = a.shape[-1]
     if align_rows_to is not None:
@@ -109,9 +120,26 @@ def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None, zero_start_inde
 _library = torch.library.Library("mslk", "FRAGMENT")
 if not hasattr(torch.ops.mslk, "quantize_fp8_row"):
     _library.define("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, int? align_rows_to=None, "
-                    "Tensor? zero_start_index_M=None) -> (Tensor, Tensor)")
+                    "Tensor? zero_start_index_M=None, float? triton_eps=None) -> (Tensor, Tensor)")
     _library.impl("quantize_fp8_row", _quantize_impl, "CUDA")
     torch.library.register_fake("mslk::quantize_fp8_row", _quantize_fp8_row_fake, lib=_library)
+
+
+_NUMERICS = "torch"
+
+
+def set_quantize_numerics(which: str) -> None:
+    """Which of the reference's two arithmetics `quantize_fp8_row` reproduces.
+
+    "torch" (default): the torch branch (fp8_quantize.py:356-378) for every call -- the bit contract this
+    package is tested against.  "triton": calls with `use_triton=True` use the arithmetic of the reference's
+    Triton kernel (fp8_quantize.py:131-207: amax clamped at `eps_opt`, scale = amax / 448, code =
+    clamp(x / scale, +-448) with IEEE divisions), as the reference does for GPU tensors; `use_triton=False`
+    still selects the torch branch."""
+    global _NUMERICS
+    if which not in ("torch", "triton"):
+        raise ValueError("quantize numerics must be 'torch' or 'triton'")
+    _NUMERICS = which
 
 
 def quantize_fp8_row(
@@ -128,15 +156,19 @@ def quantize_fp8_row(
     Returns (a_fp8 with a's shape [last dim padded to align_rows_to], scale with shape a.shape[:-1]).
     The numerics are those of the reference's torch branch (the contract this build is checked
     against bit for bit): amax is clamped at 1e-12 in the input dtype, so `eps_opt` -- which only the
-    reference's Triton branch reads -- has no effect; `use_triton` is accepted and ignored (there is one
-    implementation).  With `zero_start_index_M` (one entry per [N, K] matrix of the input viewed as
+    reference's Triton branch reads -- has no effect, and `use_triton` is ignored, unless
+    `set_quantize_numerics("triton")` was called (then `use_triton=True` selects the Triton kernel's arithmetic
+    with `eps_opt`, as the reference does on a GPU).  With `zero_start_index_M` (one entry per [N, K] matrix of the input viewed as
     [B, M, N, K]) the rows n >= zero_start_index_M[b, m] are not read and quantize like all-zero rows
     (fp8_quantize.py:123-129).
     The input must live on a GPU: there is no CPU implementation in this package.
     """
     if not a.is_cuda:
         raise RuntimeError("mslk_amd.quantize_fp8_row: input must be a GPU tensor (no CPU implementation)")
-    a_fp8, a_scale = torch.ops.mslk.quantize_fp8_row(a, scale_ub, align_rows_to, zero_start_index_M)
+    triton_eps = None
+    if _NUMERICS == "triton" and use_triton:
+        triton_eps = eps_opt if eps_opt is not None else 1e-12   # get_fp8_constants() eps (fp8_quantize.py:243-247)
+    a_fp8, a_scale = torch.ops.mslk.quantize_fp8_row(a, scale_ub, align_rows_to, zero_start_index_M, triton_eps)
     if output_device is not None and torch.device(output_device) != a.device:
         a_fp8, a_scale = a_fp8.to(output_device), a_scale.to(output_device)
     return a_fp8, a_scale

@@ -11,6 +11,8 @@ Every function restates, in plain CPU torch, the arithmetic of one reference fun
   dequant_matmul          test/gemm/triton/fp8_gemm_test.py:126-132     (tight GEMM oracle)
   matmul_fp8_row_cpu      mslk/gemm/triton/fp8_gemm.py:1186-1201        (CPU fallback = timed CPU baseline)
   grouped_*               test/gemm/triton/grouped_gemm_test.py:116-121, bench/gemm/gemm_ops.py:632-644
+  quantize_fp8_row_triton_arithmetic  mslk/quantize/triton/fp8_quantize.py:131-207 (parity unpinned at bit
+                          level: the Triton kernel cannot run here; closed forms only)
   quantize_fp8_row_jagged mslk/quantize/triton/fp8_quantize.py:123-129,236-243
   dequantize_fp8_row[_bf16] mslk/quantize/triton/fp8_quantize.py:1060-1113
   preshuffle_b            mslk/quantize/shuffle.py:182-246
@@ -66,6 +68,22 @@ def quantize_fp8_row(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None
 def dequantize_fp8_row(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
     """fp32 dequantization xq * scale[:, None] (fp8_quantize.py:1140-1182 semantics)."""
     return xq.to(torch.float32) * x_scale.to(torch.float32).reshape(*xq.shape[:-1], 1)
+
+
+def quantize_fp8_row_triton_arithmetic(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None,
+                                       eps: float = 1.0 / 512.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The arithmetic written in the reference's Triton kernel (fp8_quantize.py:131-207; eps_opt default
+    1/512, lines 215,246-247), restated with IEEE fp32 operations:
+        amax = clamp(max|a| (taken in a's dtype), eps [, scale_ub]);  scale = amax / 448 (div_rn);
+        code = e4m3fn_rne(clamp(a.f32 / scale (div_rn), -448, 448)).
+    The Triton kernel itself cannot be executed here, so this restatement is pinned only by closed forms."""
+    amax = a.abs().amax(dim=-1).to(torch.float32)
+    amax = torch.clamp(amax, min=eps)
+    if scale_ub is not None:
+        amax = torch.minimum(amax, scale_ub.reshape(-1)[0].to(torch.float32))
+    scale = amax / torch.tensor(FP8_MAX, dtype=torch.float32)
+    q = torch.clamp(a.to(torch.float32) / scale[..., None], -FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
+    return q, scale
 
 
 def dequantize_fp8_row_bf16(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:

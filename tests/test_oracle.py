@@ -329,3 +329,33 @@ def test_preshuffle_layout_by_brute_force():
                     assert flat_out[gi, pos] == flat_src[gi, n, k]
     # it is a permutation: sorting recovers the input
     assert torch.equal(out.reshape(-1).sort().values, src.reshape(-1))
+
+
+def test_triton_arithmetic_closed_forms():
+    # amax = 448 * 2^k: scale = 2^k and every x / 2^k is converted as is
+    for k in (-3, 0, 5):
+        y = (torch.tensor([[448.0, -224.0, 1.0, 0.0, 17.0, -0.4375]]) * 2.0 ** k).bfloat16()
+        q, sc = O.quantize_fp8_row_triton_arithmetic(y)
+        assert sc.item() == 2.0 ** k
+        assert q.view(torch.uint8).tolist() == [[0x7E, 0xF6, 0x38, 0x00, 0x58, 0xAE]]
+    # zero row: amax is raised to eps = 1/512 -> scale = 2^-9 / 448
+    q, sc = O.quantize_fp8_row_triton_arithmetic(torch.zeros(1, 8).bfloat16())
+    assert (q.view(torch.uint8) == 0).all() and sc.item() == (torch.tensor(2.0 ** -9) / torch.tensor(448.0)).item()
+    # rows below eps are quantized against eps, not against their own maximum: 2^-12 / (2^-9 / 448) = 56
+    q, sc = O.quantize_fp8_row_triton_arithmetic(torch.tensor([[2.0 ** -12, -2.0 ** -13]]).bfloat16())
+    assert q.float().tolist() == [[56.0, -28.0]]
+    # scale_ub below the maximum saturates (the torch branch produces NaN codes there)
+    y = torch.tensor([[100.0, -50.0, 25.0, 10.0]]).bfloat16()
+    q, sc = O.quantize_fp8_row_triton_arithmetic(y, torch.tensor([25.0]))
+    assert sc.item() == (torch.tensor(25.0) / torch.tensor(448.0)).item()
+    assert q.view(torch.uint8)[0, :3].tolist() == [0x7E, 0xFE, 0x7E] and q.float()[0, 3].item() == 176.0
+    qt, _ = O.quantize_fp8_row(y, torch.tensor([25.0]))
+    assert torch.isnan(qt.float()[0, 0])
+    # the two arithmetics agree except in the last place of a few codes
+    g = torch.Generator().manual_seed(10)
+    a = torch.randn(64, 512, generator=g).bfloat16()
+    q1, s1 = O.quantize_fp8_row_triton_arithmetic(a)
+    q2, s2 = O.quantize_fp8_row(a)
+    assert torch.allclose(s1, s2, rtol=3e-7, atol=0)
+    diff = (q1.view(torch.uint8).int() - q2.view(torch.uint8).int()).abs()
+    assert diff.max() <= 1 and (diff != 0).float().mean() < 1e-2

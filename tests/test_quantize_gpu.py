@@ -219,3 +219,43 @@ def test_dequantize_round_trip_full_size():
     xq2, s2 = mslk_amd.quantize_fp8_row(back.bfloat16())
     back2 = mslk_amd.dequantize_fp8_row(xq2, s2).float()
     assert (back2 - back).abs().max() <= back.abs().max() * 2.0 ** -7
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_triton_arithmetic_mode(dtype):
+    """`set_quantize_numerics("triton")`: codes and scales equal the oracle's restatement of the reference's
+    Triton kernel bit for bit (IEEE divisions on both sides), over the reference's shape sweep, eps variants,
+    scale_ub, jagged rows and padding; the default mode is unaffected."""
+    g = torch.Generator().manual_seed(17)
+    mslk_amd.set_quantize_numerics("triton")
+    try:
+        for shape in [(1, 16), (7, 777), (64, 1024), (2500, 4096), (3, 5, 136), (5, 20000)]:
+            a = (torch.randn(shape, generator=g) * 3).to(dtype)
+            a.view(-1, shape[-1])[0].zero_()                        # a zero row: the eps clamp decides
+            a.view(-1, shape[-1])[-1].mul_(2.0 ** -14)               # a row below 1/512
+            for eps_opt, ub in [(1.0 / 512.0, None), (None, None), (1e-4, 1.2345), (1.0 / 512.0, 1200.0)]:
+                ubt = None if ub is None else torch.tensor([ub], dtype=torch.float32)
+                xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), scale_ub=None if ubt is None else ubt.to(DEV), eps_opt=eps_opt)
+                torch.cuda.synchronize()
+                rq, rs = O.quantize_fp8_row_triton_arithmetic(a, ubt, eps_opt if eps_opt is not None else 1e-12)
+                assert torch.equal(codes(xq), codes(rq)), (shape, eps_opt, ub)
+                assert torch.equal(bits32(s), bits32(rs)), (shape, eps_opt, ub)
+        # use_triton=False keeps the torch branch
+        a = torch.randn(33, 256, generator=g).to(dtype)
+        xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), use_triton=False)
+        assert_quant_bit_exact(a, xq, s)
+        # jagged + padding
+        a = torch.randn(4, 6, 40, generator=g).to(dtype)
+        zs = torch.tensor([6, 0, 3, 1])
+        xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=zs.to(DEV), align_rows_to=16)
+        masked = a.clone()
+        for gi in range(4):
+            masked[gi, int(zs[gi]):] = 0
+        rq, rs = O.quantize_fp8_row_triton_arithmetic(masked)
+        assert torch.equal(codes(xq)[..., :40], codes(rq)) and (codes(xq)[..., 40:] == 0).all()
+        assert torch.equal(bits32(s), bits32(rs))
+    finally:
+        mslk_amd.set_quantize_numerics("torch")
+    a = torch.randn(8, 64, generator=g).to(dtype)
+    xq, s = mslk_amd.quantize_fp8_row(a.to(DEV))
+    assert_quant_bit_exact(a, xq, s)
