@@ -114,11 +114,16 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (!dense_tiled_supports(p)) return hipErrorInvalidValue;
   // 256 x 256 tiles once they give every CU work; 128 x 128 below that.
   const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
+  // 128 x 128 tiles: with at most one tile per CU a workgroup gets the whole LDS for a five-deep ring (its step is
+  // much shorter than a memory round trip); with more tiles two workgroups per CU hide each other's latency better.
+  const int64_t small_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
   if (p.w_preshuffled) {
     if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
+    if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
     return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
   }
   if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false>(p, s);
   return launch_tiled_shape<TileShape<128, 128>, false>(p, s);
 }
 

@@ -30,8 +30,12 @@ namespace mslk_amd {
 
 constexpr int kBK = 128;  // bytes (= fp8 elements) of K per main-loop step
 
-template <int BM, int BN, int WAVES_M = 2, int WAVES_N = 2>
+// RING = 0: two XQ buffers and three WQ buffers (weights two steps ahead, activations one).
+// RING = n: n buffers for each operand, both streams n - 1 steps ahead -- for small tiles, whose step is much
+// shorter than a memory round trip.
+template <int BM, int BN, int WAVES_M = 2, int WAVES_N = 2, int RING_STAGES = 0>
 struct TileShape {
+  static constexpr int RING = RING_STAGES;
   static constexpr int kBM = BM, kBN = BN;
   static constexpr int WM = WAVES_M, WN = WAVES_N;   // wave grid over the tile
   static constexpr int NW = WAVES_M * WAVES_N;
@@ -40,8 +44,8 @@ struct TileShape {
   static constexpr int FN = BN / WAVES_N / 16;  // 16-row n fragments per wave
   static constexpr int A_BYTES = BM * kBK;
   static constexpr int B_BYTES = BN * kBK;
-  static constexpr int A_STAGES = 2;            // XQ tiles: the one being read and the one in flight
-  static constexpr int B_STAGES = 3;            // WQ tiles: one being read, two in flight
+  static constexpr int A_STAGES = RING_STAGES ? RING_STAGES : 2;   // XQ tiles: the one being read and the one in flight
+  static constexpr int B_STAGES = RING_STAGES ? RING_STAGES : 3;   // WQ tiles: one being read, two in flight
   static constexpr int LDS_BYTES = A_STAGES * A_BYTES + B_STAGES * B_BYTES;
   static constexpr int LA = BM / 8 / NW;        // wave-level loads of the A tile per wave per step
   static constexpr int LB = BN / 8 / NW;
@@ -199,10 +203,11 @@ struct GemmTile {
   // all its LDS reads have returned, then passes the workgroup barrier.
   template <int PENDING>
   MSLK_AMD_DEVINL static void wait_and_barrier() {
-    static_assert(PENDING >= 0 && PENDING < 16, "vmcnt immediate");
+    static_assert(PENDING >= 0 && PENDING < 64, "vmcnt is a 6-bit counter");
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");                  // no LDS access moves across the barrier at compile time
-    __builtin_amdgcn_s_waitcnt(0x0070 | PENDING);   // vmcnt(PENDING) lgkmcnt(0), expcnt untouched
+    // vmcnt(PENDING) lgkmcnt(0), expcnt untouched; vmcnt is split into bits [3:0] and [15:14] of the immediate
+    __builtin_amdgcn_s_waitcnt(0x0070 | (PENDING & 15) | ((PENDING >> 4) << 14));
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_sched_barrier(0);
@@ -222,9 +227,11 @@ struct GemmTile {
   //     each XQ fragment is re-loaded from `a_nxt` right after the MFMA that used it last, so the barrier
   //     and the LDS latency overlap with matrix work and the following step starts with its first
   //     fragments already on their way.
-  template <bool DMA_A, bool DMA_B, bool NEXT>
-  MSLK_AMD_DEVINL void step(const char* b_cur, char* a_nxt, const char* b_nxt, char* b_far, int k_a, int k_b,
-                            v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
+  // In the symmetric ring (TileShape::RING) the XQ loads go to `a_dst` != `a_nxt` as well, and PENDING, the
+  // number of this wave's youngest loads that may still be in flight at the barrier, covers RING - 2 steps.
+  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING>
+  MSLK_AMD_DEVINL void step(const char* b_cur, char* a_dst, const char* a_nxt, const char* b_nxt, char* b_far, int k_a,
+                            int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
     constexpr int HALF = TS::FN / 2;
     static_assert((TS::LA + TS::LB) % HALF == 0, "DMA loads spread evenly over the first half");
     constexpr int NDMA = (TS::LA + TS::LB) / HALF;   // DMA loads per MFMA group
@@ -248,7 +255,7 @@ struct GemmTile {
         if (tn < HALF && d >= 0) {
           const int q = tn * NDMA + d;   // all XQ loads are older than all WQ loads of the step
           if (q < TS::LA) {
-            if constexpr (DMA_A) issue_a(a_nxt, k_a, q);
+            if constexpr (DMA_A) issue_a(a_dst, k_a, q);
           } else {
             if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
           }
@@ -259,7 +266,7 @@ struct GemmTile {
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (NEXT) {
-      wait_and_barrier<DMA_B ? TS::LB : 0>();
+      wait_and_barrier<PENDING>();
       wf0 = load_frag_b(b_tile_of(b_nxt), 0, fo);
     }
     const char* a_next = a_tile_of(a_nxt);
@@ -285,53 +292,99 @@ struct GemmTile {
   MSLK_AMD_DEVINL void run(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, const float* xs,
                            const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K,
                            uint32_t ld) {
-    init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
     v4f acc[TS::FN][TS::FM];
+    accumulate(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+  }
+
+  // K loop only: acc = sum over the K bytes of the operand rows starting at xq_tile / wq_tile.  Ends with a
+  // workgroup barrier, after which the LDS buffers are dead.
+  MSLK_AMD_DEVINL void accumulate(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
+                                  uint32_t ld, v4f (&acc)[TS::FN][TS::FM]) {
+    init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
 #pragma unroll
     for (int tn = 0; tn < TS::FN; ++tn)
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) acc[tn][tm] = v4f{0.f, 0.f, 0.f, 0.f};
 
-    char* a_cur = lds;
-    char* a_nxt = lds + TS::A_BYTES;
-    char* b_cur = lds + 2 * TS::A_BYTES;
-    char* b_nxt = b_cur + TS::B_BYTES;
-    char* b_far = b_nxt + TS::B_BYTES;
     const int KT = K / kBK;           // full steps
     const int k_tail = K - KT * kBK;  // 0 or a multiple of 16
     v8i xf[TS::FM], wf0;
-    if (KT > 0) {
-      issue_a_all(a_cur, 0);
-      issue_b_all(b_cur, 0);
-      if (KT > 1) {
-        issue_b_all(b_nxt, kBK);
-        wait_and_barrier<TS::LB>();
-      } else {
-        wait_and_barrier<0>();
+    char* a_tail = lds;               // buffers the K tail may use once the full steps are done
+    char* b_tail = lds + TS::A_STAGES * TS::A_BYTES;
+    if constexpr (TS::RING == 0) {
+      char* a_cur = lds;
+      char* a_nxt = lds + TS::A_BYTES;
+      char* b_cur = lds + 2 * TS::A_BYTES;
+      char* b_nxt = b_cur + TS::B_BYTES;
+      char* b_far = b_nxt + TS::B_BYTES;
+      if (KT > 0) {
+        issue_a_all(a_cur, 0);
+        issue_b_all(b_cur, 0);
+        if (KT > 1) {
+          issue_b_all(b_nxt, kBK);
+          wait_and_barrier<TS::LB>();
+        } else {
+          wait_and_barrier<0>();
+        }
+        load_first_frags(a_cur, b_cur, xf, wf0);
+        // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
+        for (int kt = 0; kt < KT - 2; ++kt) {
+          step<true, true, true, TS::LB>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
+          { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
+          { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
+        }
+        if (KT > 1) {
+          step<true, false, true, 0>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
+          { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
+          { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
+        }
+        step<false, false, false, 0>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
       }
-      load_first_frags(a_cur, b_cur, xf, wf0);
-      // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
-      for (int kt = 0; kt < KT - 2; ++kt) {
-        step<true, true, true>(b_cur, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
-        { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
-        { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
+    } else {
+      // Symmetric ring: buffer i % RING holds step i; step kt fetches step kt + RING - 1 into the buffers step
+      // kt - 1 used (free since the barrier of that step), and at its barrier everything but the loads of the
+      // last RING - 2 steps has to be there.
+      constexpr int NS = TS::RING;
+      constexpr int PER_STEP = TS::LA + TS::LB;
+      static_assert(NS >= 3 && (NS - 2) * PER_STEP < 64, "vmcnt is a 6-bit counter");
+      char* const a0 = lds;
+      char* const b0 = lds + NS * TS::A_BYTES;
+      auto abuf = [&](int i) { return a0 + i * TS::A_BYTES; };
+      auto bbuf = [&](int i) { return b0 + i * TS::B_BYTES; };
+      if (KT > 0) {
+        const int pre = KT < NS - 1 ? KT : NS - 1;
+        for (int i = 0; i < pre; ++i) {
+          issue_a_all(abuf(i), i * kBK);
+          issue_b_all(bbuf(i), i * kBK);
+        }
+        if (pre == NS - 1) wait_and_barrier<(NS - 2) * PER_STEP>();
+        else wait_and_barrier<0>();
+        load_first_frags(abuf(0), bbuf(0), xf, wf0);
+        int cur = 0;   // kt % NS
+        int kt = 0;
+        for (; kt + NS - 1 < KT; ++kt) {
+          const int nxt = cur + 1 == NS ? 0 : cur + 1, far = cur == 0 ? NS - 1 : cur - 1;
+          step<true, true, true, (NS - 2) * PER_STEP>(bbuf(cur), abuf(far), abuf(nxt), bbuf(nxt), bbuf(far),
+                                                       (kt + NS - 1) * kBK, (kt + NS - 1) * kBK, acc, xf, wf0);
+          cur = nxt;
+        }
+        for (; kt + 1 < KT; ++kt) {   // nothing left to fetch: the first of these steps waits for all that is in flight
+          const int nxt = cur + 1 == NS ? 0 : cur + 1;
+          step<false, false, true, 0>(bbuf(cur), abuf(nxt), abuf(nxt), bbuf(nxt), bbuf(nxt), 0, 0, acc, xf, wf0);
+          cur = nxt;
+        }
+        step<false, false, false, 0>(bbuf(cur), abuf(cur), abuf(cur), bbuf(cur), bbuf(cur), 0, 0, acc, xf, wf0);
       }
-      if (KT > 1) {
-        step<true, false, true>(b_cur, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
-        { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
-        { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
-      }
-      step<false, false, false>(b_cur, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
     }
     if (k_tail > 0) {
       __syncthreads();   // everybody is done with the buffers of the full steps before one pair is refilled
-      issue_loads_tail(a_nxt, b_nxt, KT * kBK, k_tail);
+      issue_loads_tail(a_tail, b_tail, KT * kBK, k_tail);
       __syncthreads();
-      load_first_frags(a_nxt, b_nxt, xf, wf0);
-      step<false, false, false>(b_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
+      load_first_frags(a_tail, b_tail, xf, wf0);
+      step<false, false, false, 0>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
     }
     __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
-    epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
   }
 
   // Epilogue.  A lane's accumulators of one 16-row m fragment are 4 consecutive n in each of the
