@@ -117,12 +117,19 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // 128 x 128 tiles: with at most one tile per CU a workgroup gets the whole LDS for a five-deep ring (its step is
   // much shorter than a memory round trip); with more tiles two workgroups per CU hide each other's latency better.
   const int64_t small_tiles = (int64_t)((p.M + 127) / 128) * ((p.N + 127) / 128);
+  // At most 128 / 64 such tiles: narrower tiles (128 x 64, 128 x 32; four waves stacked along M, six / eight ring
+  // buffers) put the weight stream on two / four times as many CUs, still one workgroup per CU; the activations they
+  // re-read come from L2.  Going narrower than one workgroup per CU was measured and is slower.
   if (p.w_preshuffled) {
     if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
+    if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, true>(p, s);
+    if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, true>(p, s);
     if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
     return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
   }
   if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false>(p, s);
+  if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false>(p, s);
   if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false>(p, s);
   return launch_tiled_shape<TileShape<128, 128>, false>(p, s);
 }

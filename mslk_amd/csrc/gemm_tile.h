@@ -235,7 +235,8 @@ struct GemmTile {
     constexpr int HALF = TS::FN / 2;
     static_assert((TS::LA + TS::LB) % HALF == 0, "DMA loads spread evenly over the first half");
     constexpr int NDMA = (TS::LA + TS::LB) / HALF;   // DMA loads per MFMA group
-    static_assert(NDMA <= TS::FM, "one DMA per MFMA slot");
+    constexpr int PER_SLOT = (NDMA + TS::FM - 1) / TS::FM;            // 1 unless the tile has few MFMAs per group
+    constexpr int SLOTS = (NDMA + PER_SLOT - 1) / PER_SLOT;          // MFMA slots of a group that carry loads
     const FragOff fo = frag_off();
     const char* b_tile = b_tile_of(b_cur);
     v8i wf = wf0;
@@ -251,13 +252,18 @@ struct GemmTile {
       for (int tm = 0; tm < TS::FM; ++tm) {
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
         if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
-        const int d = tm - (TS::FM - NDMA);
+        const int d = tm - (TS::FM - SLOTS);
         if (tn < HALF && d >= 0) {
-          const int q = tn * NDMA + d;   // all XQ loads are older than all WQ loads of the step
-          if (q < TS::LA) {
-            if constexpr (DMA_A) issue_a(a_dst, k_a, q);
-          } else {
-            if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
+#pragma unroll
+          for (int j = 0; j < PER_SLOT; ++j) {
+            const int q = tn * NDMA + d * PER_SLOT + j;   // all XQ loads are older than all WQ loads of the step
+            if (d * PER_SLOT + j < NDMA) {
+              if (q < TS::LA) {
+                if constexpr (DMA_A) issue_a(a_dst, k_a, q);
+              } else {
+                if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
+              }
+            }
           }
         }
         __builtin_amdgcn_sched_barrier(0);

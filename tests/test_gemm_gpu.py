@@ -307,3 +307,24 @@ def test_seeded_random_shape_sweep():
         ref = O.dequant_matmul(xq, wq, xs, ws, None if bias is None else bias.float())
         assert y.shape == (M, N)
         assert_gemm_close(y, ref, f"case {case}: {M}x{N}x{K} bias={None if bias is None else bias.dtype} op={op}")
+
+
+@pytest.mark.parametrize("M,N,K", [(65, 8192, 8192), (128, 4096, 4096), (200, 2048, 4096), (256, 1024, 8192), (100, 520, 2064),
+                                   (384, 4096, 2048), (128, 1024, 14336), (96, 16384, 2048), (130, 64, 272), (70, 136, 144),
+                                   (512, 8192, 1024), (66, 72, 16)])
+def test_medium_m_shapes_use_narrow_and_ring_tiles(M, N, K):
+    """Shapes between the skinny kernel (M <= 64) and a full grid of 256 x 256 tiles: 128 x 32 / 128 x 64 / 128 x 128
+    tiles with deep operand rings.  Oracle tolerance, both output types, bias, and the pre-shuffled weights."""
+    g = torch.Generator().manual_seed(M * 3 + N + K)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    bias = (torch.randn(N, generator=g) * 0.5).float()
+    d = _gpu(xq, wq, xs, ws)
+    y = torch.ops.mslk.f8f8bf16_rowwise(*d, bias=bias.to(DEV))
+    y16 = torch.ops.mslk.f8f8f16_rowwise(*d)
+    torch.cuda.synchronize()
+    assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws, bias), f"{M}x{N}x{K}")
+    assert_gemm_close(y16, O.dequant_matmul(xq, wq, xs, ws), f"fp16 {M}x{N}x{K}")
+    if N % 16 == 0 and K % 64 == 0:
+        yp = torch.ops.mslk.f8f8bf16_rowwise_preshuffle(d[0], mslk_amd.preshuffle_b_mfma(d[1]), d[2], d[3], bias=bias.to(DEV))
+        torch.cuda.synchronize()
+        assert_gemm_close(yp, O.dequant_matmul(xq, wq, xs, ws, bias), f"pre-shuffled {M}x{N}x{K}")
