@@ -228,6 +228,20 @@ def main():
         extras["gemm_cfg1_graph_replay"] = {"ms": graph_ms, "TFLOPs": flops / (graph_ms * 1e-3) / 1e12,
                                             "frac_mfma": flops / (graph_ms * 1e-3) / PEAK_FP8_FLOPS,
                                             "note": "120 launches in one HIP graph, same operand rotation"}
+        if not args.no_extras and args.only == "":
+            # For scale only: the vendor library (hipBLASLt behind torch._scaled_mm, row-wise scales) on the same
+            # operand rotation.  Not part of the product path and not a fallback.
+            try:
+                def vendor_step(i):
+                    xq, wq, xs, ws, y = sets[i % NSETS]
+                    torch._scaled_mm(xq, wq.t(), scale_a=xs[:, None], scale_b=ws[None, :], out_dtype=torch.bfloat16, out=y)
+                for i in range(20):
+                    vendor_step(i)
+                v_ms = _median_events_ms(vendor_step, 100)
+                extras["vendor_scaled_mm_rowwise_cfg1"] = {"ms": v_ms, "TFLOPs": flops / (v_ms * 1e-3) / 1e12,
+                                                           "note": "torch._scaled_mm (hipBLASLt), same operands"}
+            except Exception as e:  # the library may not offer row-wise scales for this shape
+                extras["vendor_scaled_mm_rowwise_cfg1"] = {"error": str(e)[:160]}
         if args.only == "gemm":
             print(json.dumps({"gemm_ms": kern_ms, "tflops": achieved, "graph_ms": graph_ms,
                               "graph_tflops": flops / (graph_ms * 1e-3) / 1e12}))

@@ -7,20 +7,26 @@ namespace mslk_amd {
 namespace {
 
 constexpr int kXcds = 8;      // MI355X: 8 accelerator dies, workgroups are dealt to them round-robin
+constexpr int kCus = 256;     // compute units; a 256 x 256 tile takes the whole LDS of one
 constexpr int kGroupM = 4;    // tiles of one XCD form kGroupM-row panels (L2 reuse of the WQ panel)
 
 // Workgroup id -> tile.  Consecutive workgroup ids land on different XCDs (each with a private
 // L2), so XCD x is handed a contiguous range of the panel-ordered tile list.
-MSLK_AMD_DEVINL bool map_tile(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
-  const int ntiles = tiles_m * tiles_n;
-  const int per_xcd = (ntiles + kXcds - 1) / kXcds;
-  const int t = (bid % kXcds) * per_xcd + bid / kXcds;
-  if (t >= ntiles || bid / kXcds >= per_xcd) return false;
+// Entry t of the panel-ordered tile list.
+MSLK_AMD_DEVINL void list_tile(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int panel = kGroupM * tiles_n;
   const int first_m = (t / panel) * kGroupM;
   const int rows = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
   tm = first_m + (t % panel) % rows;
   tn = (t % panel) / rows;
+}
+
+MSLK_AMD_DEVINL bool map_tile(int bid, int tiles_m, int tiles_n, int& tm, int& tn) {
+  const int ntiles = tiles_m * tiles_n;
+  const int per_xcd = (ntiles + kXcds - 1) / kXcds;
+  const int t = (bid % kXcds) * per_xcd + bid / kXcds;
+  if (t >= ntiles || bid / kXcds >= per_xcd) return false;
+  list_tile(t, tiles_m, tiles_n, tm, tn);
   return true;
 }
 
@@ -38,6 +44,71 @@ __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p
   if constexpr (BIAS == 2) bias = reinterpret_cast<const uint16_t*>(p.bias) + n0;
   tile.run(lds, p.xq + (int64_t)m0 * p.K, p.wq + (int64_t)n0 * p.K, p.xs + m0, p.ws + n0, bias,
            p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K);
+}
+
+// More tiles than CUs: one workgroup per CU walks its share of the tile list (XCD x keeps its contiguous slice,
+// its workgroups take the entries round-robin, so at any time an XCD works on neighbouring tiles as it does with
+// one workgroup per tile).  The first DMA loads of the next tile are issued before the epilogue of the current one
+// and land while it runs, and no workgroup has to be started per tile.
+template <typename TS, int BIAS, bool PS>
+__global__ __launch_bounds__(TS::NTHREADS) void dense_persistent_kernel(GemmProblem p, int tiles_m, int tiles_n) {
+  static_assert(TS::RING == 0 && TS::NTHREADS == 256, "two-plus-three buffer tiles with four waves");
+  constexpr int BM = TS::kBM, BN = TS::kBN;
+  using Tile = GemmTile<TS, BIAS, PS>;
+  // The epilogue parks its transposes in the two buffers the next tile's prologue does not fill.
+  static_assert(2 * Tile::EPI_WAVE_BYTES <= TS::A_BYTES && 2 * Tile::EPI_WAVE_BYTES <= TS::B_BYTES, "transpose buffers fit");
+  __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
+  const int ntiles = tiles_m * tiles_n;
+  const int per_xcd = (ntiles + kXcds - 1) / kXcds;
+  const int xcd = blockIdx.x % kXcds, stride = gridDim.x / kXcds;
+  int j = blockIdx.x / kXcds;
+  if (j >= per_xcd || xcd * per_xcd + j >= ntiles) return;
+  Tile tile;
+  tile.out_f16 = p.out_f16;
+  const int wave = Tile::wave_id();
+  char* const epi_buf = lds + (wave < 2 ? TS::A_BYTES + wave * Tile::EPI_WAVE_BYTES
+                                        : 2 * TS::A_BYTES + 2 * TS::B_BYTES + (wave - 2) * Tile::EPI_WAVE_BYTES);
+  int tm, tn;
+  list_tile(xcd * per_xcd + j, tiles_m, tiles_n, tm, tn);
+  tm = __builtin_amdgcn_readfirstlane(tm);   // the divisions above ran on the vector unit; the results are uniform
+  tn = __builtin_amdgcn_readfirstlane(tn);
+  tile.prologue(lds, p.xq + (int64_t)tm * BM * p.K, p.wq + (int64_t)tn * BN * p.K, p.M - tm * BM, p.N - tn * BN, p.K,
+                (uint32_t)p.K);
+  for (;;) {
+    v4f acc[TS::FN][TS::FM];
+    tile.template accumulate_issued<true>(lds, p.K, acc);
+    const int m0 = tm * BM, n0 = tn * BN;
+    j += stride;
+    const bool more = j < per_xcd && xcd * per_xcd + j < ntiles;
+    if (more) {
+      list_tile(xcd * per_xcd + j, tiles_m, tiles_n, tm, tn);
+      tm = __builtin_amdgcn_readfirstlane(tm);
+      tn = __builtin_amdgcn_readfirstlane(tn);
+      tile.prologue(lds, p.xq + (int64_t)tm * BM * p.K, p.wq + (int64_t)tn * BN * p.K, p.M - tm * BM, p.N - tn * BN, p.K,
+                    (uint32_t)p.K);
+    }
+    const void* bias = nullptr;
+    if constexpr (BIAS == 1) bias = reinterpret_cast<const float*>(p.bias) + n0;
+    if constexpr (BIAS == 2) bias = reinterpret_cast<const uint16_t*>(p.bias) + n0;
+    tile.epilogue_at(epi_buf, acc, p.xs + m0, p.ws + n0, bias, p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N);
+    if (!more) break;
+    // The per-lane load offsets of the next tile are formed again here rather than carried through the epilogue,
+    // which needs the registers.
+    tile.init(p.xq + (int64_t)tm * BM * p.K, p.wq + (int64_t)tn * BN * p.K, p.M - tm * BM < BM ? p.M - tm * BM : BM,
+              p.N - tn * BN < BN ? p.N - tn * BN : BN, (uint32_t)p.K);
+  }
+}
+
+template <typename TS, bool PS>
+hipError_t launch_persistent_shape(const GemmProblem& p, int wgs, hipStream_t s) {
+  constexpr int BM = TS::kBM, BN = TS::kBN;
+  const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  switch (p.bias_dtype) {
+    case 0: dense_persistent_kernel<TS, 0, PS><<<wgs, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    case 1: dense_persistent_kernel<TS, 1, PS><<<wgs, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    default: dense_persistent_kernel<TS, 2, PS><<<wgs, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+  }
+  return hipGetLastError();
 }
 
 template <typename TS, bool PS>
@@ -105,14 +176,15 @@ __global__ void fill_zero_kernel(uint16_t* y, int64_t n) {
 
 bool dense_tiled_supports(const GemmProblem& p) {
   if (p.w_preshuffled && (p.N % 16 != 0 || p.K % 64 != 0)) return false;   // the blocked layout itself needs this
-  return p.K % 16 == 0 && p.K >= 16 && (int64_t)256 * p.K < (int64_t(1) << 32) &&
+  return p.K % 16 == 0 && p.K >= 16 && (int64_t)256 * p.K < (int64_t(1) << 32) && p.N < (1 << 26) &&
          reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0 &&
          reinterpret_cast<uintptr_t>(p.y) % 16 == 0;
 }
 
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (!dense_tiled_supports(p)) return hipErrorInvalidValue;
-  // 256 x 256 tiles once they give every CU work; 128 x 128 below that.
+  // 256 x 256 tiles once they give every CU work (one persistent workgroup per CU when there are more tiles than
+  // CUs); 128 x 128 below that.
   const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
   // 128 x 128 tiles: with at most one tile per CU a workgroup gets the whole LDS for a five-deep ring (its step is
   // much shorter than a memory round trip); with more tiles two workgroups per CU hide each other's latency better.
@@ -121,12 +193,14 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // buffers) put the weight stream on two / four times as many CUs, still one workgroup per CU; the activations they
   // re-read come from L2.  Going narrower than one workgroup per CU was measured and is slower.
   if (p.w_preshuffled) {
+    if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, true>(p, kCus, s);
     if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
     if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, true>(p, s);
     if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, true>(p, s);
     if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
     return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
   }
+  if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, kCus, s);
   if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
   if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false>(p, s);
   if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false>(p, s);

@@ -274,7 +274,7 @@ hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s) {
 
 // Whether every operand row of the problem can be fetched by the 16-byte DMA path.
 static bool device_groups_aligned(const DeviceGroups& p) {
-  return p.K % 16 == 0 && (int64_t)256 * p.K < (int64_t(1) << 32) &&
+  return p.K % 16 == 0 && (int64_t)256 * p.K < (int64_t(1) << 32) && p.N < (1 << 26) &&
          reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0;
 }
 

@@ -60,8 +60,11 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 
 // The output is written once and not re-read by this kernel: a streaming (non-temporal) store keeps
 // it from displacing the operand tiles in L2 and from piling up as dirty lines to flush at kernel end.
+// Written as an instruction with vector-register operands: given the choice, the register allocator parks the
+// read-back values in accumulator registers, all of which hold the tile, and spills part of it.
 MSLK_AMD_DEVINL void store16_stream(uint16_t* dst, uint4 val) {
-  __builtin_nontemporal_store(v4i{(int)val.x, (int)val.y, (int)val.z, (int)val.w}, reinterpret_cast<v4i*>(dst));
+  const v4i v = {(int)val.x, (int)val.y, (int)val.z, (int)val.w};
+  asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
 }
 
 MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
@@ -86,7 +89,9 @@ struct GemmTile {
   // xq/wq point at row m0 / n0 of the operands; rows_a / rows_b = valid rows from there (>= 1).
   // `ld` = bytes between consecutive rows of XQ and of WQ (equal to K unless the operands are K slices).
   MSLK_AMD_DEVINL void init(const uint8_t* xq_tile, const uint8_t* wq_tile, int rows_a, int rows_b, uint32_t ld) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int lane = threadIdx.x & 63;
+    asm volatile("" : "+v"(lane));   // recompute the row / chunk of each load per tile instead of keeping 32 values live
+    const int wave = wave_id();
     a_base = xq_tile;
     b_base = wq_tile;
 #pragma unroll
@@ -137,7 +142,7 @@ struct GemmTile {
   // K tail (K % 128 != 0, K % 16 == 0): only `k_valid` bytes of each row remain.  Chunks at or
   // beyond K are zero-filled with a plain LDS store by the lane that would have fetched them.
   MSLK_AMD_DEVINL void issue_loads_tail(char* abuf, char* bbuf, int k0, int k_valid) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63, wave = wave_id();
 #pragma unroll
     for (int i = 0; i < TS::LA; ++i) {
       const int row = (wave * TS::LA + i) * 8 + (lane >> 3);
@@ -307,7 +312,34 @@ struct GemmTile {
   // workgroup barrier, after which the LDS buffers are dead.
   MSLK_AMD_DEVINL void accumulate(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
                                   uint32_t ld, v4f (&acc)[TS::FN][TS::FM]) {
+    if constexpr (TS::RING == 0) {
+      prologue(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld);
+    } else {
+      init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
+    }
+    accumulate_issued<false>(lds, K, acc);
+  }
+
+  // Two-plus-three buffers only: per-lane addresses of a tile and the first DMA loads of its K loop (step 0 of both
+  // operands, step 1 of WQ) into the buffers the loop starts from.  A persistent workgroup calls this for its next
+  // tile before the epilogue of the current one, which must then stay out of those three buffers.
+  MSLK_AMD_DEVINL void prologue(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
+                                uint32_t ld) {
+    static_assert(TS::RING == 0, "the symmetric ring issues its own prologue");
     init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
+    const int KT = K / kBK;
+    if (KT > 0) {
+      issue_a_all(lds, 0);
+      issue_b_all(lds + 2 * TS::A_BYTES, 0);
+      if (KT > 1) issue_b_all(lds + 2 * TS::A_BYTES + TS::B_BYTES, kBK);
+    }
+  }
+
+  // K loop after prologue() (or, for the symmetric ring, after init()).  DRAIN: the wave has other memory
+  // operations in flight behind the prologue loads (the stores of the previous tile's epilogue), so the first wait
+  // is for all of them instead of "all but the youngest WQ loads".
+  template <bool DRAIN>
+  MSLK_AMD_DEVINL void accumulate_issued(char* lds, int K, v4f (&acc)[TS::FN][TS::FM]) {
 #pragma unroll
     for (int tn = 0; tn < TS::FN; ++tn)
 #pragma unroll
@@ -325,14 +357,8 @@ struct GemmTile {
       char* b_nxt = b_cur + TS::B_BYTES;
       char* b_far = b_nxt + TS::B_BYTES;
       if (KT > 0) {
-        issue_a_all(a_cur, 0);
-        issue_b_all(b_cur, 0);
-        if (KT > 1) {
-          issue_b_all(b_nxt, kBK);
-          wait_and_barrier<TS::LB>();
-        } else {
-          wait_and_barrier<0>();
-        }
+        if (KT > 1 && !DRAIN) wait_and_barrier<TS::LB>();
+        else wait_and_barrier<0>();
         load_first_frags(a_cur, b_cur, xf, wf0);
         // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
         for (int kt = 0; kt < KT - 2; ++kt) {
@@ -399,8 +425,16 @@ struct GemmTile {
   // private LDS buffer (row pitch BN + 16 bytes keeps the 8-byte writes and 16-byte reads off shared
   // banks), then reads it back row-major so that one store instruction writes 4 full rows of
   // BN/2 bf16 (16 lanes x 16 bytes each).
+  // LDS the epilogue of one wave uses: two transpose buffers and the row scales of the wave's rows
+  static constexpr int EPI_WAVE_BYTES = 2 * 16 * ((TS::kBN / TS::WN) * 2 + 16) + (TS::kBM / TS::WM) * 4;
   MSLK_AMD_DEVINL void epilogue(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                 const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
+    static_assert((TS::NTHREADS / 64) * EPI_WAVE_BYTES <= TS::LDS_BYTES && EPI_WAVE_BYTES % 16 == 0, "epilogue buffers fit");
+    epilogue_at(lds + wave_id() * EPI_WAVE_BYTES, acc, xs, ws, bias, y, m_rem, n_rem, N);
+  }
+  // As epilogue(), with the wave's private transpose buffer (EPI_WAVE_BYTES) placed by the caller.
+  MSLK_AMD_DEVINL void epilogue_at(char* buf, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
+                                   const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     // Tiles whose columns are all valid (the common case, also for the ragged last row tile of an MoE
     // group) take a path whose only bounds logic is one row test per store instruction.
     // 16-byte accesses need 16-byte aligned rows of Y and aligned scale / bias vectors (a tile that
@@ -409,27 +443,32 @@ struct GemmTile {
     const bool full = n_rem >= TS::kBN && vec16 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
                       (BIAS == 0 || (reinterpret_cast<uintptr_t>(bias) & (BIAS == 1 ? 15 : 7)) == 0);
     if (out_f16) {
-      if (full) epilogue_impl<true, true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
-      else epilogue_impl<false, true>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      if (full) epilogue_impl<true, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else epilogue_impl<false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
     } else {
-      if (full) epilogue_impl<true, false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
-      else epilogue_impl<false, false>(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      if (full) epilogue_impl<true, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else epilogue_impl<false, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
     }
   }
 
   // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged.
   template <bool FULL, bool F16>
-  MSLK_AMD_DEVINL void epilogue_impl(char* lds, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
+  MSLK_AMD_DEVINL void epilogue_impl(char* buf, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                      const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     constexpr int WN = TS::kBN / TS::WN;         // columns per wave
     constexpr int PITCH = WN * 2 + 16;           // bytes per staged row
     constexpr int BUF = 16 * PITCH;
     constexpr int CH = WN / 8;                   // 16-byte chunks per row (16 for BN = 256)
     constexpr int RPI = 64 / CH;                 // rows written per store instruction
-    const int lane = threadIdx.x & 63, wave = wave_id();
+    int lane = threadIdx.x & 63;
+    // Everything derived from the lane id below is recomputed per call: inside a loop over tiles the compiler would
+    // otherwise keep these values live across the K loop, where registers are scarce, and spill them.
+    asm volatile("" : "+v"(lane));
+    const int wave = wave_id();
     const int wm = wave / TS::WN, wn = wave % TS::WN;
     const int j = lane & 15, q = lane >> 4;
-    char* buf = lds + wave * 2 * BUF;
+    constexpr int ROWS_W = TS::kBM / TS::WM;     // rows per wave
+    static_assert(2 * BUF + ROWS_W * 4 == EPI_WAVE_BYTES, "epilogue buffer size");
     const int n_base = wn * WN;
     const int m_base = wm * (TS::kBM / TS::WM);
     const bool vec_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
@@ -465,13 +504,21 @@ struct GemmTile {
     }
 
     const int rd_row = lane / CH, rd_chunk = lane % CH;
+    const uint32_t lane_off = ((uint32_t)rd_row * (uint32_t)N + (uint32_t)(n_base + rd_chunk * 8)) * 2u;   // bytes; 16 N < 2^31
+    constexpr int NP = 16 / RPI;                 // store instructions per 16-row fragment
+
+    // The row scales go through LDS (one global load per row instead of one per lane and fragment row, and no
+    // registers held for the whole epilogue).  All global loads of the epilogue are issued before its first store: the
+    // wait for a load issued between stores would also wait for every older store to be acknowledged by memory.
+    float* xs_lds = reinterpret_cast<float*>(buf + 2 * BUF);
 #pragma unroll
-    for (int tm = 0; tm < TS::FM; ++tm) {
+    for (int r = lane; r < ROWS_W; r += 64) xs_lds[r] = m_base + r < m_rem ? xs[m_base + r] : 0.f;
+
+    // Scale, convert and park n fragments [tn0, tn1) of fragment row tm in transpose buffer tm & 1.
+    auto park = [&](int tm, int tn0, int tn1, float xsv) {
       char* b = buf + (tm & 1) * BUF;
-      const int m = m_base + tm * 16 + j;
-      const float xsv = m < m_rem ? xs[m] : 0.f;
 #pragma unroll
-      for (int tn = 0; tn < TS::FN; ++tn) {
+      for (int tn = tn0; tn < tn1; ++tn) {
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
@@ -483,17 +530,63 @@ struct GemmTile {
         pk.y = pack_out_x2<F16>(v[2], v[3]);
         *reinterpret_cast<uint2*>(b + j * PITCH + (tn * 16 + 4 * q) * 2) = pk;
       }
-      // the buffer is private to the wave: LDS operations of one wave complete in order
+    };
+    // Row-major read-back of fragment row tm (the buffer is private to the wave and LDS operations of one wave
+    // complete in order, so no barrier separates it from park(tm)).
+    auto fetch = [&](int tm, uint4 (&val)[NP]) {
+      const char* b = buf + (tm & 1) * BUF;
 #pragma unroll
-      for (int pass = 0; pass < 16 / RPI; ++pass) {
-        const int row = pass * RPI + rd_row;
-        const uint4 val = *reinterpret_cast<const uint4*>(b + row * PITCH + rd_chunk * 16);
-        const int mm = m_base + tm * 16 + row;
-        const int nn = n_base + rd_chunk * 8;
-        uint16_t* dst = y + (int64_t)mm * N + nn;
-        if constexpr (FULL) {
-          if (mm < m_rem) store16_stream(dst, val);
-        } else {
+      for (int pass = 0; pass < NP; ++pass)
+        val[pass] = *reinterpret_cast<const uint4*>(b + (pass * RPI + rd_row) * PITCH + rd_chunk * 16);
+    };
+    // Wave-uniform 64-bit row base + one 32-bit lane offset that is the same for every store of the tile.
+    auto dst_of = [&](int tm, int pass) {
+      return reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(y + (int64_t)(m_base + tm * 16 + pass * RPI) * N) + lane_off);
+    };
+
+    if constexpr (FULL) {
+      // With one wave per SIMD nothing else hides the LDS round trip between parking a fragment row and
+      // storing it, so the rows are pipelined by hand: the read-back of row tm - 1 is issued before the
+      // arithmetic of row tm and its stores follow that arithmetic.
+      // The stores of row tm - 1 are spread between the pieces of that arithmetic, so the store path and the
+      // vector ALU work side by side.
+      static_assert(TS::FN % NP == 0, "whole n fragments per store");
+      uint4 val[NP];
+      // consecutive store instructions of a wave are RPI rows apart: one 64-bit add per store
+      char* dst = reinterpret_cast<char*>(y + (int64_t)m_base * N) + lane_off;
+      const int64_t dst_step = (int64_t)RPI * N * 2;
+      float xsv = xs_lds[j];
+#pragma unroll
+      for (int tm = 0; tm <= TS::FM; ++tm) {
+        if (tm > 0) fetch(tm - 1, val);
+        const float xsv_next = tm + 1 < TS::FM ? xs_lds[(tm + 1) * 16 + j] : 0.f;   // read one fragment row ahead
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pass = 0; pass < NP; ++pass) {
+          if (tm < TS::FM) park(tm, pass * (TS::FN / NP), (pass + 1) * (TS::FN / NP), xsv);
+          __builtin_amdgcn_sched_barrier(0);
+          if (tm > 0) {
+            const int r0 = m_base + (tm - 1) * 16 + pass * RPI;   // first of the RPI rows this instruction writes
+            if (r0 + RPI <= m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);           // wave-uniform test
+            else if (r0 + rd_row < m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);    // ragged last rows
+            dst += dst_step;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        xsv = xsv_next;
+      }
+    } else {
+#pragma unroll
+      for (int tm = 0; tm < TS::FM; ++tm) {
+        park(tm, 0, TS::FN, xs_lds[tm * 16 + j]);
+        uint4 vals[NP];
+        fetch(tm, vals);
+#pragma unroll
+        for (int pass = 0; pass < NP; ++pass) {
+          const uint4 val = vals[pass];
+          const int mm = m_base + tm * 16 + pass * RPI + rd_row;
+          const int nn = n_base + rd_chunk * 8;
+          uint16_t* dst = dst_of(tm, pass);
           if (mm >= m_rem || nn >= n_rem) continue;
           if (vec_store && nn + 7 < n_rem) {
             store16_stream(dst, val);
