@@ -328,3 +328,27 @@ def test_medium_m_shapes_use_narrow_and_ring_tiles(M, N, K):
         yp = torch.ops.mslk.f8f8bf16_rowwise_preshuffle(d[0], mslk_amd.preshuffle_b_mfma(d[1]), d[2], d[3], bias=bias.to(DEV))
         torch.cuda.synchronize()
         assert_gemm_close(yp, O.dequant_matmul(xq, wq, xs, ws, bias), f"pre-shuffled {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(4352, 4352, 256), (4100, 4500, 400), (8192, 2304, 128), (2304, 8200, 48), (5000, 4608, 144)])
+def test_more_tiles_than_compute_units(M, N, K):
+    """More than 256 tiles of 256 x 256: one persistent workgroup per CU walks several tiles, fetching the next
+    tile's first operands before the epilogue of the current one.  Ragged last rows / columns, K tails, one-step and
+    zero-step K loops, both bias types, both output types and the pre-shuffled weights against the oracle."""
+    assert ((M + 255) // 256) * ((N + 255) // 256) > 256
+    g = torch.Generator().manual_seed(M + 7 * N + K)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    bias = (torch.randn(N, generator=g) * 0.5).float()
+    d = _gpu(xq, wq, xs, ws)
+    y = torch.ops.mslk.f8f8bf16_rowwise(*d, bias=bias.to(DEV))
+    yb = torch.ops.mslk.f8f8bf16_rowwise(*d, bias=bias.bfloat16().to(DEV))
+    y16 = torch.ops.mslk.f8f8f16_rowwise(*d)
+    torch.cuda.synchronize()
+    ref = O.dequant_matmul(xq, wq, xs, ws)
+    assert_gemm_close(y, ref + bias, f"{M}x{N}x{K}")
+    assert_gemm_close(yb, ref + bias.bfloat16().float(), f"bf16 bias {M}x{N}x{K}")
+    assert_gemm_close(y16, ref, f"fp16 {M}x{N}x{K}")
+    if N % 16 == 0 and K % 64 == 0:
+        yp = torch.ops.mslk.f8f8bf16_rowwise_preshuffle(d[0], mslk_amd.preshuffle_b_mfma(d[1]), d[2], d[3])
+        torch.cuda.synchronize()
+        assert_gemm_close(yp, ref, f"pre-shuffled {M}x{N}x{K}")
