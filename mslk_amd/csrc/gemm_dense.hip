@@ -79,7 +79,7 @@ __global__ __launch_bounds__(TS::NTHREADS) void dense_persistent_kernel(GemmProb
     tile.template accumulate_issued<true>(lds, p.K, acc);
     const int m0 = tm * BM, n0 = tn * BN;
     j += stride;
-    const bool more = j < per_xcd && xcd * per_xcd + j < ntiles;
+    const bool more = __builtin_amdgcn_readfirstlane((int)(j < per_xcd && xcd * per_xcd + j < ntiles)) != 0;
     if (more) {
       list_tile(xcd * per_xcd + j, tiles_m, tiles_n, tm, tn);
       tm = __builtin_amdgcn_readfirstlane(tm);

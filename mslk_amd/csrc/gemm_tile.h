@@ -61,10 +61,12 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // The output is written once and not re-read by this kernel: a streaming (non-temporal) store keeps
 // it from displacing the operand tiles in L2 and from piling up as dirty lines to flush at kernel end.
 // Written as an instruction with vector-register operands: given the choice, the register allocator parks the
-// read-back values in accumulator registers, all of which hold the tile, and spills part of it.
+// read-back values in accumulator registers, all of which hold the tile, and spills part of it.  The compiler does
+// not see a store here, so the wait states the hardware needs between a store of more than 8 bytes and a vector
+// instruction that overwrites its data registers (the allocator reuses them at once) are part of the statement.
 MSLK_AMD_DEVINL void store16_stream(uint16_t* dst, uint4 val) {
   const v4i v = {(int)val.x, (int)val.y, (int)val.z, (int)val.w};
-  asm volatile("global_store_dwordx4 %0, %1, off nt" : : "v"(dst), "v"(v) : "memory");
+  asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
 }
 
 MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
@@ -442,17 +444,21 @@ struct GemmTile {
     const bool vec16 = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     const bool full = n_rem >= TS::kBN && vec16 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
                       (BIAS == 0 || (reinterpret_cast<uintptr_t>(bias) & (BIAS == 1 ? 15 : 7)) == 0);
+    const bool interior = full && m_rem >= TS::kBM;   // no bounds logic at all
     if (out_f16) {
-      if (full) epilogue_impl<true, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
-      else epilogue_impl<false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      if (interior) epilogue_impl<true, true, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else if (full) epilogue_impl<true, true, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else epilogue_impl<false, true, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
     } else {
-      if (full) epilogue_impl<true, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
-      else epilogue_impl<false, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      if (interior) epilogue_impl<true, false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else if (full) epilogue_impl<true, false, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+      else epilogue_impl<false, false, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
     }
   }
 
-  // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged.
-  template <bool FULL, bool F16>
+  // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged unless
+  // ALL_ROWS says that the tile has all its rows too.
+  template <bool FULL, bool F16, bool ALL_ROWS>
   MSLK_AMD_DEVINL void epilogue_impl(char* buf, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                      const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     constexpr int WN = TS::kBN / TS::WN;         // columns per wave
@@ -506,13 +512,19 @@ struct GemmTile {
     const int rd_row = lane / CH, rd_chunk = lane % CH;
     const uint32_t lane_off = ((uint32_t)rd_row * (uint32_t)N + (uint32_t)(n_base + rd_chunk * 8)) * 2u;   // bytes; 16 N < 2^31
     constexpr int NP = 16 / RPI;                 // store instructions per 16-row fragment
+    constexpr bool ACC_IN_AGPRS = TS::FM * TS::FN * 4 >= 256;
+    if constexpr (ACC_IN_AGPRS) {
+      // The reads below are opaque to the compiler's hazard handling: let the last MFMAs of the K loop retire
+      // (16 passes each) before their results are read.
+      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15");
+    }
 
     // The row scales go through LDS (one global load per row instead of one per lane and fragment row, and no
     // registers held for the whole epilogue).  All global loads of the epilogue are issued before its first store: the
     // wait for a load issued between stores would also wait for every older store to be acknowledged by memory.
     float* xs_lds = reinterpret_cast<float*>(buf + 2 * BUF);
 #pragma unroll
-    for (int r = lane; r < ROWS_W; r += 64) xs_lds[r] = m_base + r < m_rem ? xs[m_base + r] : 0.f;
+    for (int r = lane; r < ROWS_W; r += 64) xs_lds[r] = (ALL_ROWS || m_base + r < m_rem) ? xs[m_base + r] : 0.f;
 
     // Scale, convert and park n fragments [tn0, tn1) of fragment row tm in transpose buffer tm & 1.
     auto park = [&](int tm, int tn0, int tn1, float xsv) {
@@ -522,7 +534,13 @@ struct GemmTile {
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-          v[r] = (acc[tn][tm][r] * xsv) * wsv[tn][r];
+          // A tile of 256 accumulators per lane stays in accumulator registers until this point: left to itself
+          // the register allocator moves part of it to vector registers ahead of time, runs out of them and spills,
+          // and a reload between the stores waits for all of them.  (Smaller tiles live in vector registers.)
+          float a;
+          if constexpr (ACC_IN_AGPRS) asm("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[tn][tm][r]));
+          else a = acc[tn][tm][r];
+          v[r] = (a * xsv) * wsv[tn][r];
           if constexpr (BIAS != 0) v[r] += bv[tn][r];
         }
         uint2 pk;
@@ -567,7 +585,7 @@ struct GemmTile {
           __builtin_amdgcn_sched_barrier(0);
           if (tm > 0) {
             const int r0 = m_base + (tm - 1) * 16 + pass * RPI;   // first of the RPI rows this instruction writes
-            if (r0 + RPI <= m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);           // wave-uniform test
+            if (ALL_ROWS || r0 + RPI <= m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);   // wave-uniform test
             else if (r0 + rd_row < m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);    // ragged last rows
             dst += dst_step;
           }
