@@ -538,7 +538,7 @@ struct GemmTile {
           // the register allocator moves part of it to vector registers ahead of time, runs out of them and spills,
           // and a reload between the stores waits for all of them.  (Smaller tiles live in vector registers.)
           float a;
-          if constexpr (ACC_IN_AGPRS) asm("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[tn][tm][r]));
+          if constexpr (ACC_IN_AGPRS) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[tn][tm][r]));   // volatile: stays behind the s_nop
           else a = acc[tn][tm][r];
           v[r] = (a * xsv) * wsv[tn][r];
           if constexpr (BIAS != 0) v[r] += bv[tn][r];
