@@ -7,7 +7,22 @@ namespace mslk_amd {
 namespace {
 
 constexpr int kXcds = 8;      // MI355X: 8 accelerator dies, workgroups are dealt to them round-robin
-constexpr int kCus = 256;     // compute units; a 256 x 256 tile takes the whole LDS of one
+constexpr int kCus = 256;     // compute units of a whole MI355X; a 256 x 256 tile takes the whole LDS of one
+
+// Compute units of the current device (a partitioned MI355X shows fewer than 256), as a multiple of the XCD count:
+// the number of persistent workgroups.  Queried once per device.
+int persistent_workgroups() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kCus;
+  if (cached[dev] == 0) {
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = kCus;
+    cus = cus / kXcds * kXcds;
+    cached[dev] = cus < kXcds ? kXcds : cus;
+  }
+  return cached[dev];
+}
 constexpr int kGroupM = 4;    // tiles of one XCD form kGroupM-row panels (L2 reuse of the WQ panel)
 
 // Workgroup id -> tile.  Consecutive workgroup ids land on different XCDs (each with a private
@@ -193,14 +208,14 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // buffers) put the weight stream on two / four times as many CUs, still one workgroup per CU; the activations they
   // re-read come from L2.  Going narrower than one workgroup per CU was measured and is slower.
   if (p.w_preshuffled) {
-    if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, true>(p, kCus, s);
+    if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, true>(p, persistent_workgroups(), s);
     if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
     if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, true>(p, s);
     if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, true>(p, s);
     if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
     return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
   }
-  if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, kCus, s);
+  if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, persistent_workgroups(), s);
   if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
   if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false>(p, s);
   if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false>(p, s);

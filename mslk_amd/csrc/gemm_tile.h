@@ -524,7 +524,10 @@ struct GemmTile {
     // wait for a load issued between stores would also wait for every older store to be acknowledged by memory.
     float* xs_lds = reinterpret_cast<float*>(buf + 2 * BUF);
 #pragma unroll
-    for (int r = lane; r < ROWS_W; r += 64) xs_lds[r] = (ALL_ROWS || m_base + r < m_rem) ? xs[m_base + r] : 0.f;
+    for (int i = 0; i < (ROWS_W + 63) / 64; ++i) {
+      const int r = lane + i * 64;
+      if (ROWS_W % 64 == 0 || r < ROWS_W) xs_lds[r] = (ALL_ROWS || m_base + r < m_rem) ? xs[m_base + r] : 0.f;
+    }
 
     // Scale, convert and park n fragments [tn0, tn1) of fragment row tm in transpose buffer tm & 1.
     auto park = [&](int tm, int tn0, int tn1, float xsv) {
