@@ -162,11 +162,11 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
     return fail("%s: pre-shuffled weights need N %% 16 == 0 and K %% 64 == 0 (got N=%lld, K=%lld)", op, (long long)N, (long long)K);
   GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
                 (int)M, (int)N, (int)K, bias_dtype, out_f16, preshuffled};
-  // M <= 64: the weight-streaming kernel, except where wide weights give the narrow-tile kernel a full grid and
-  // its shared activation tiles win (measured crossovers: M > 32 at N >= 8192, M > 16 at N >= 16384).
+  // M <= 64: the weight-streaming kernel, except on wide row-major weights, where short tiles that share their
+  // activation rows through LDS win from M = 9 on (measured crossover at N = 8192 ... 28672).  Pre-shuffled weights
+  // keep the streaming kernel, whose register-direct weight loads stay ahead up to M = 64.
   const bool tiled_ok = dense_tiled_supports(p);
-  // Pre-shuffled weights keep the streaming kernel, whose register-direct weight loads stay ahead up to M = 64.
-  const bool wide = !p.w_preshuffled && ((p.M > 32 && p.N >= 8192) || (p.M > 16 && p.N >= 16384));
+  const bool wide = !p.w_preshuffled && p.M > 8 && p.N >= 8192;
   if (skinny_supports(p) && !(tiled_ok && wide)) return check_hip(launch_skinny(p, s), "skinny launch");
   if (tiled_ok) return check_hip(launch_dense_tiled(p, s), "tiled launch");
   return check_hip(launch_generic(p, s), "generic launch");

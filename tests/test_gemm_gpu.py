@@ -352,3 +352,20 @@ def test_more_tiles_than_compute_units(M, N, K):
         yp = torch.ops.mslk.f8f8bf16_rowwise_preshuffle(d[0], mslk_amd.preshuffle_b_mfma(d[1]), d[2], d[3])
         torch.cuda.synchronize()
         assert_gemm_close(yp, ref, f"pre-shuffled {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(9, 8192, 1024), (16, 8200, 512), (32, 16384, 384), (24, 20000, 272), (33, 8192, 2048),
+                                   (48, 12296, 144), (64, 9000, 1040), (64, 16383, 128), (40, 28672, 256), (17, 8192, 16)])
+def test_small_m_on_wide_weights_uses_short_tiles(M, N, K):
+    """8 < M <= 64 with N >= 8192 and row-major weights: 32 x 32 and 64 x 32 tiles (two- and four-wave workgroups, deep
+    operand rings) instead of the weight-streaming kernel.  Ragged rows and columns, K tails, bias, fp16 output."""
+    g = torch.Generator().manual_seed(M * 5 + N + K)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    bias = (torch.randn(N, generator=g) * 0.5).float()
+    d = _gpu(xq, wq, xs, ws)
+    y = torch.ops.mslk.f8f8bf16_rowwise(*d, bias=bias.to(DEV))
+    y16 = torch.ops.mslk.f8f8f16_rowwise(*d)
+    torch.cuda.synchronize()
+    ref = O.dequant_matmul(xq, wq, xs, ws)
+    assert_gemm_close(y, ref + bias, f"{M}x{N}x{K}")
+    assert_gemm_close(y16, ref, f"fp16 {M}x{N}x{K}")
