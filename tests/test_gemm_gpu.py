@@ -140,7 +140,7 @@ def test_unaligned_views_take_the_generic_path():
     assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws))
 
 
-@pytest.mark.parametrize("M,N,K", [(512, 1024, 512), (16, 1024, 1024)])
+@pytest.mark.parametrize("M,N,K", [(512, 1024, 512), (16, 1024, 1024), (4352, 4352, 128), (16, 8192, 256), (64, 8192, 256)])
 def test_hip_graph_capture_and_replay(M, N, K):
     """The reference tests capture + replay (test/gemm/gemm_test.py:440-447); replay several times with
     eager work in between and compare every replay with the eager result."""
