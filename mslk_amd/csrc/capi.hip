@@ -163,10 +163,10 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
   GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
                 (int)M, (int)N, (int)K, bias_dtype, out_f16, preshuffled};
   // M <= 64: the weight-streaming kernel, except on wide row-major weights, where short tiles that share their
-  // activation rows through LDS win from M = 9 on (measured crossover at N = 8192 ... 28672).  Pre-shuffled weights
+  // activation rows through LDS win from M = 9 on.  Pre-shuffled weights
   // keep the streaming kernel, whose register-direct weight loads stay ahead up to M = 64.
   const bool tiled_ok = dense_tiled_supports(p);
-  const bool wide = !p.w_preshuffled && p.M > 8 && p.N >= 8192;
+  const bool wide = !p.w_preshuffled && p.M > 8 && p.N >= kShortTileMinN;
   if (skinny_supports(p) && !(tiled_ok && wide)) return check_hip(launch_skinny(p, s), "skinny launch");
   if (tiled_ok) return check_hip(launch_dense_tiled(p, s), "tiled launch");
   return check_hip(launch_generic(p, s), "generic launch");

@@ -218,8 +218,8 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // M <= 64 on wide row-major weights (the caller sends M <= 8 to the weight-streaming kernel): the activation rows
   // are re-read by every workgroup, so the tile is only as tall as M needs -- 32 x 32 (two waves) or 64 x 32 tiles with
   // six to eight ring buffers, two workgroups per CU.  Measured against the 128-row tiles and the streaming kernel
-  // at N = 8192 ... 28672.
-  if (p.M <= 64 && p.N >= 8192) {
+  // at N = 5120 ... 28672.
+  if (p.M <= 64 && p.N >= kShortTileMinN) {
     if (p.M <= 32 && p.N <= 16384) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false>(p, s);
     if (p.M <= 32 || p.N < 16384) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false>(p, s);
   }

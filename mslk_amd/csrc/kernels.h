@@ -61,6 +61,9 @@ struct GemmProblem {
 bool dense_tiled_supports(const GemmProblem& p);
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s);
 bool skinny_supports(const GemmProblem& p);
+// Row-major weights at least this wide take the short LDS tiles instead of the weight-streaming kernel for 8 < M <= 64
+// (measured crossover: streaming wins at N = 4096, tiles from N = 5120 on).
+constexpr int kShortTileMinN = 5120;
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s);
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s);   // any shape, slow
 hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s);

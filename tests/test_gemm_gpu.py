@@ -355,9 +355,10 @@ def test_more_tiles_than_compute_units(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(9, 8192, 1024), (16, 8200, 512), (32, 16384, 384), (24, 20000, 272), (33, 8192, 2048),
-                                   (48, 12296, 144), (64, 9000, 1040), (64, 16383, 128), (40, 28672, 256), (17, 8192, 16)])
+                                   (48, 12296, 144), (64, 9000, 1040), (64, 16383, 128), (40, 28672, 256), (17, 8192, 16),
+                                   (12, 5120, 1024), (64, 6152, 400), (31, 7168, 2048)])
 def test_small_m_on_wide_weights_uses_short_tiles(M, N, K):
-    """8 < M <= 64 with N >= 8192 and row-major weights: 32 x 32 and 64 x 32 tiles (two- and four-wave workgroups, deep
+    """8 < M <= 64 with N >= 5120 and row-major weights: 32 x 32 and 64 x 32 tiles (two- and four-wave workgroups, deep
     operand rings) instead of the weight-streaming kernel.  Ragged rows and columns, K tails, bias, fp16 output."""
     g = torch.Generator().manual_seed(M * 5 + N + K)
     xq, wq, xs, ws = _random_problem(M, N, K, g)
