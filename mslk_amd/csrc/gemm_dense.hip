@@ -1,5 +1,6 @@
 // Dense f8f8bf16_rowwise for gfx950: LDS-tiled MFMA kernel (large shapes), a generic
 // any-shape kernel, and the zero-fill used for empty problems.
+#include <atomic>
 #include "gemm_tile.h"
 #include "kernels.h"
 
@@ -12,16 +13,17 @@ constexpr int kCus = 256;     // compute units of a whole MI355X; a 256 x 256 ti
 // Compute units of the current device (a partitioned MI355X shows fewer than 256), as a multiple of the XCD count:
 // the number of persistent workgroups.  Queried once per device.
 int persistent_workgroups() {
-  static int cached[64] = {};
+  static std::atomic<int> cached[64];   // zero-initialised; concurrent first calls store the same value
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kCus;
-  if (cached[dev] == 0) {
-    int cus = 0;
+  int cus = cached[dev].load(std::memory_order_relaxed);
+  if (cus == 0) {
     if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = kCus;
     cus = cus / kXcds * kXcds;
-    cached[dev] = cus < kXcds ? kXcds : cus;
+    if (cus < kXcds) cus = kXcds;
+    cached[dev].store(cus, std::memory_order_relaxed);
   }
-  return cached[dev];
+  return cus;
 }
 constexpr int kGroupM = 4;    // tiles of one XCD form kGroupM-row panels (L2 reuse of the WQ panel)
 
