@@ -19,10 +19,14 @@
 //     WQ tiles of steps k+1 and k+2 are in flight (the weights are the cold, read-once stream).
 // Math
 //   * v_mfma_f32_16x16x128_f8f6f4 (both operands e4m3, unit block scales).  WQ rows are the first
-//     operand and XQ rows the second, so a lane ends up holding 4 consecutive n for one m and
-//     stores them as one 8-byte bf16x4.
+//     operand and XQ rows the second, so a lane ends up holding 4 consecutive n for one m.
 //   * Both operands give lane (i = l & 15, g = l >> 4) the 32 bytes k in [32 g, 32 g + 32) of
 //     row i; any k permutation would do as long as both operands share it.
+// Epilogue
+//   * A wave has its SIMD to itself, so every instruction and every memory wait of the epilogue is exposed.  Scales
+//     and bias are fetched before the first store (a load waited for between stores waits for the stores too); each
+//     16-row fragment row is scaled, converted and transposed through a wave-private LDS buffer, and the read-back
+//     and the stores of one fragment row are interleaved with the arithmetic of the next.
 #pragma once
 #include "common.h"
 
