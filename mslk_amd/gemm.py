@@ -449,7 +449,12 @@ def _fake_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_accu
 
 
 def _fake_grouped(XQ, WQ, x_scale, w_scale):
-    return [torch.empty((x.shape[0], w.shape[0]), dtype=torch.bfloat16, device=x.device) for x, w in zip(XQ, WQ)]
+    # as the kernel (and the reference): views into one flat buffer
+    if len(XQ) == 0:
+        return []
+    sizes = [x.shape[0] * w.shape[0] for x, w in zip(XQ, WQ)]
+    flat = torch.empty(sum(sizes), dtype=torch.bfloat16, device=XQ[0].device)
+    return [t.view(x.shape[0], w.shape[0]) for t, x, w in zip(flat.split(sizes), XQ, WQ)]
 
 
 def _fake_grouped_cat(XQ, WQ, x_scale, w_scale):

@@ -1,0 +1,69 @@
+"""torch.library.opcheck on the registered ops: the fake (meta) kernels agree with the real ones in shape, dtype,
+strides and device (the reference registers fake kernels
+for the same purpose, mslk/gemm/_meta.py:26-65,114-126 and mslk/quantize/triton/fp8_quantize.py:381-407)."""
+import pytest
+import torch
+
+import mslk_amd  # noqa: F401
+from mslk_amd import moe  # noqa: F401
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+F8 = torch.float8_e4m3fn
+CHECKS = ("test_faketensor",)   # the schema checker multiplies tensors, which float8 does not implement
+
+
+def _codes(*shape):
+    return torch.randint(0, 0x58, shape, dtype=torch.uint8, device=DEV).view(F8)
+
+
+def test_opcheck_quantize_and_dequantize():
+    x = torch.randn(48, 256, device=DEV, dtype=torch.bfloat16)
+    torch.library.opcheck(torch.ops.mslk.quantize_fp8_row, (x,), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.mslk.quantize_fp8_row, (x, torch.tensor([1200.0], device=DEV), 64), test_utils=CHECKS)
+    q, s = torch.ops.mslk.quantize_fp8_row(x)
+    torch.library.opcheck(torch.ops.mslk.dequantize_fp8_row, (q, s), test_utils=CHECKS)
+
+
+def test_opcheck_dense_family():
+    M, N, K = 80, 96, 256
+    xq, wq = _codes(M, K), _codes(N, K)
+    xs, ws = torch.rand(M, device=DEV) + 0.5, torch.rand(N, device=DEV) + 0.5
+    bias = torch.randn(N, device=DEV)
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise, (xq, wq, xs, ws), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise, (xq, wq, xs, ws, bias), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.mslk.f8f8f16_rowwise, (xq, wq, xs, ws), test_utils=CHECKS)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_out, (xq, wq, xs, ws, out), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_batched,
+                          (_codes(3, M, K), _codes(3, N, K), torch.rand(3, M, device=DEV), torch.rand(3, N, device=DEV)),
+                          test_utils=CHECKS)
+
+
+def test_opcheck_grouped_family():
+    G, N, K = 3, 64, 128
+    sizes = [5, 0, 40]
+    M = sum(sizes)
+    xq, wq = _codes(M, K), _codes(G, N, K)
+    xs, ws = torch.rand(M, device=DEV) + 0.5, torch.rand(G, N, device=DEV) + 0.5
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked,
+                          (xq, wq, xs, ws, torch.tensor(sizes, dtype=torch.int64, device=DEV)), test_utils=CHECKS)
+    ends = torch.tensor(sizes, device=DEV).cumsum(0).to(torch.int32)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)   # the reference's schema takes the output tensor
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_grouped_mm, (xq, wq, xs, ws, ends, out), test_utils=CHECKS)
+    # the TensorList op keeps the reference's check that N and K are at least 512
+    xq2, wq2 = _codes(M, 512), _codes(G, 512, 512)
+    ws2 = torch.rand(G, 512, device=DEV) + 0.5
+    xl, sl = list(xq2.split(sizes)), list(xs.split(sizes))
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_grouped, (xl, list(wq2), sl, list(ws2)), test_utils=CHECKS)
+
+
+def test_opcheck_fused_producers():
+    T, D, E = 24, 256, 4
+    x = torch.randn(T, 2 * D, device=DEV, dtype=torch.bfloat16)
+    torch.library.opcheck(torch.ops.mslk.silu_mul_quant, (x[:, :D], x[:, D:]), test_utils=CHECKS)
+    tok = torch.randperm(T, device=DEV).to(torch.int32)
+    exp = torch.randint(0, E, (T,), device=DEV)
+    scores = torch.rand(T, E, device=DEV)
+    torch.library.opcheck(torch.ops.mslk.gather_scale_quant_dense_tokens, (x[:, :D].contiguous(), tok, exp, scores),
+                          test_utils=CHECKS)
