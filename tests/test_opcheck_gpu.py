@@ -67,3 +67,37 @@ def test_opcheck_fused_producers():
     scores = torch.rand(T, E, device=DEV)
     torch.library.opcheck(torch.ops.mslk.gather_scale_quant_dense_tokens, (x[:, :D].contiguous(), tok, exp, scores),
                           test_utils=CHECKS)
+
+
+def test_opcheck_preshuffle_dynamic_and_cat():
+    M, N, K = 48, 64, 128
+    xq, wq = _codes(M, K), _codes(N, K)
+    xs, ws = torch.rand(M, device=DEV) + 0.5, torch.rand(N, device=DEV) + 0.5
+    wps = mslk_amd.preshuffle_b_mfma(wq)
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_preshuffle, (xq, wps, xs, ws), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.mslk.f8f8f16_rowwise_preshuffle, (xq, wps, xs, ws), test_utils=CHECKS)
+    G = 3
+    xq3, wq3 = _codes(G, M, 512), _codes(G, 512, 512)          # the reference's check: N and K at least 512
+    xs3, ws3 = torch.rand(G, M, device=DEV) + 0.5, torch.rand(G, 512, device=DEV) + 0.5
+    live = torch.tensor([5, 0, 48], dtype=torch.int64, device=DEV)
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_grouped_dynamic, (xq3, wq3, xs3, ws3, live), test_utils=CHECKS)
+    sizes = [5, 0, 40]
+    xq2, wq2 = _codes(sum(sizes), 512), _codes(G, 512, 512)
+    xs2, ws2 = torch.rand(sum(sizes), device=DEV) + 0.5, torch.rand(G, 512, device=DEV) + 0.5
+    torch.library.opcheck(torch.ops.mslk.f8f8bf16_rowwise_grouped_cat,
+                          (list(xq2.split(sizes)), list(wq2), list(xs2.split(sizes)), list(ws2)), test_utils=CHECKS)
+
+
+def test_ops_trace_under_torch_compile():
+    """Dynamo + AOT autograd with fake tensors trace quantize -> GEMM into one graph (no graph breaks) and the compiled
+    function returns what the eager one does."""
+    w = torch.randn(96, 256, device=DEV, dtype=torch.bfloat16)
+    wq, ws = mslk_amd.quantize_fp8_row(w)
+
+    def linear(x):
+        xq, xs = torch.ops.mslk.quantize_fp8_row(x)
+        return torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
+
+    x = torch.randn(40, 256, device=DEV, dtype=torch.bfloat16)
+    compiled = torch.compile(linear, backend="aot_eager", fullgraph=True)
+    assert torch.equal(compiled(x), linear(x))
