@@ -40,7 +40,15 @@ _SCHEMAS = {
 _library = torch.library.Library("mslk", "FRAGMENT")
 
 
+try:   # the raw handle of the current stream without building a Stream object (4 us -> 0.3 us per call)
+    from torch._C import _cuda_getCurrentRawStream as _raw_stream
+except ImportError:   # pragma: no cover
+    _raw_stream = None
+
+
 def _stream_ptr(device: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 

@@ -16,7 +16,15 @@ FP8_DTYPE = torch.float8_e4m3fn  # gfx950 is OCP FP8 (reference: mslk/utils/devi
 _DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
 
+try:   # the raw handle of the current stream without building a Stream object (4 us -> 0.3 us per call)
+    from torch._C import _cuda_getCurrentRawStream as _raw_stream
+except ImportError:   # pragma: no cover
+    _raw_stream = None
+
+
 def _stream_ptr(device: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
