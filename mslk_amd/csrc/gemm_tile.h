@@ -518,8 +518,8 @@ struct GemmTile {
     constexpr int NP = 16 / RPI;                 // store instructions per 16-row fragment
     constexpr bool ACC_IN_AGPRS = TS::FM * TS::FN * 4 >= 256;
     if constexpr (ACC_IN_AGPRS) {
-      // The reads below are opaque to the compiler's hazard handling: let the last MFMAs of the K loop retire
-      // (16 passes each) before their results are read.
+      // The reads below are opaque to the compiler's hazard handling: 48 wait states let the last MFMA of the K loop
+      // (32 cycles) retire before its result is read.
       asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15");
     }
 
