@@ -370,3 +370,30 @@ def test_small_m_on_wide_weights_uses_short_tiles(M, N, K):
     ref = O.dequant_matmul(xq, wq, xs, ws)
     assert_gemm_close(y, ref + bias, f"{M}x{N}x{K}")
     assert_gemm_close(y16, ref, f"fp16 {M}x{N}x{K}")
+
+
+def test_seeded_random_sweep_small_m_wide_n():
+    """Forty seeded shapes with M <= 96 and N around and above the width from which short tiles replace the
+    weight-streaming kernel (M = 8 / 9, 32 / 33, 64 / 65; N = 4096 ... 20000; K with and without tails), row-major and
+    pre-shuffled weights, with and without bias, both output types."""
+    g = torch.Generator().manual_seed(77)
+    edges_m = [1, 8, 9, 16, 31, 32, 33, 48, 63, 64, 65, 96]
+    for case in range(40):
+        M = edges_m[case % len(edges_m)] if case % 3 else int(torch.randint(1, 97, (1,), generator=g))
+        N = int(torch.randint(4096 // 8, 20000 // 8, (1,), generator=g)) * 8
+        if case % 4 == 0:
+            N = N // 16 * 16
+        K = int(torch.randint(1, 24, (1,), generator=g)) * (64 if case % 2 else 16)
+        xq, wq, xs, ws = _random_problem(M, N, K, g)
+        bias = (torch.randn(N, generator=g) * 0.5).to(torch.bfloat16 if case % 2 else torch.float32) if case % 3 == 0 else None
+        d = _gpu(xq, wq, xs, ws)
+        ref = O.dequant_matmul(xq, wq, xs, ws, None if bias is None else bias.float())
+        op = torch.ops.mslk.f8f8f16_rowwise if case % 5 == 1 else torch.ops.mslk.f8f8bf16_rowwise
+        y = op(*d, bias=None if bias is None else bias.to(DEV))
+        torch.cuda.synchronize()
+        assert_gemm_close(y, ref, f"case {case}: {M}x{N}x{K} op={op}")
+        if N % 16 == 0 and K % 64 == 0:
+            yp = torch.ops.mslk.f8f8bf16_rowwise_preshuffle(d[0], mslk_amd.preshuffle_b_mfma(d[1]), d[2], d[3],
+                                                            bias=None if bias is None else bias.to(DEV))
+            torch.cuda.synchronize()
+            assert_gemm_close(yp, ref, f"case {case} pre-shuffled: {M}x{N}x{K}")
