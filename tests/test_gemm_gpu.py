@@ -397,3 +397,24 @@ def test_seeded_random_sweep_small_m_wide_n():
                                                             bias=None if bias is None else bias.to(DEV))
             torch.cuda.synchronize()
             assert_gemm_close(yp, ref, f"case {case} pre-shuffled: {M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 512, 1024), (300, 520, 640), (1024, 1024, 512)])
+def test_matches_the_model_level_fake_quant_statement(M, N, K):
+    """The reference states the same semantics a second time in its MoE baseline (mslk/moe/layers.py:476-488):
+    y = bf16( bf16_matmul(xq.bf16, wq.bf16^T) * xs[:, None] * ws[None, :] ).  e4m3 values are exact in bf16, so that
+    expression differs from the kernel's only by the bf16 rounding of the un-scaled matmul: one more rounding of
+    2^-9 relative."""
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    xq, xs = O.quantize_fp8_row(x)
+    wq, ws = O.quantize_fp8_row(w)
+    y = torch.ops.mslk.f8f8bf16_rowwise(*_gpu(xq, wq, xs, ws))
+    torch.cuda.synchronize()
+    stated = (torch.matmul(xq.to(torch.bfloat16), wq.to(torch.bfloat16).t()) * xs[:, None] * ws[None, :]).to(torch.bfloat16)
+    err = (y.float().cpu() - stated.float()).abs()
+    # two bf16 roundings apart at most; results that cancel to almost nothing also see the accumulation order
+    assert (err <= stated.float().abs() * 2.0 ** -7 + stated.float().abs().max() * 2.0 ** -10).all()
+    max_rel, normwise = O.gemm_errors(y.float().cpu(), stated.float())
+    assert max_rel <= O.MAX_REL_TOL and normwise <= 2 * O.NORMWISE_TOL
