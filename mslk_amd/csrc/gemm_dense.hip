@@ -228,7 +228,7 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, persistent_workgroups(), s);
   if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
   // 64 < M <= 256: 64 x 64 tiles (four waves stacked along M, five ring buffers, two workgroups per CU) wherever they
-  // cover at least as many CUs as the 128-row tiles below would, in one round: rows 65 ... 128 then do not cost a
+  // cover at least as many CUs as the 128-row tiles below would, in a single pass: rows 65 ... 128 then do not cost a
   // second, half-empty 128-row tile's worth of activation traffic (N = K = 8192, M = 96: 23.8 -> 21.2 us; N = 4096,
   // K = 14336, M = 96: 36.3 -> 30.4 us).
   if (p.M > 64 && p.M <= 256 && p.N >= 4096) {
