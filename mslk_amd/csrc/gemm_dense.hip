@@ -227,11 +227,11 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   }
   if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, persistent_workgroups(), s);
   if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
-  // 64 < M <= 256: 64 x 64 tiles (four waves stacked along M, five ring buffers, two workgroups per CU) wherever they
-  // cover at least as many CUs as the 128-row tiles below would, in a single pass: rows 65 ... 128 then do not cost a
-  // second, half-empty 128-row tile's worth of activation traffic (N = K = 8192, M = 96: 23.8 -> 21.2 us; N = 4096,
-  // K = 14336, M = 96: 36.3 -> 30.4 us).
-  if (p.M > 64 && p.M <= 256 && p.N >= 4096) {
+  // M > 64 with at most one 64 x 64 tile per CU: such tiles (four waves stacked along M, five ring buffers, two
+  // workgroups per CU) wherever they cover at least as many CUs as the 128-row tiles below would, in a single pass:
+  // rows 65 ... 128 then do not cost a second, half-empty 128-row tile's worth of activation traffic (N = K = 8192,
+  // M = 96: 23.8 -> 21.2 us; N = 4096, K = 14336, M = 96: 36.3 -> 30.4 us; 1024^3: 5.9 -> 5.5 us).
+  if (p.M > 64 && p.N >= 1024) {
     const int64_t tiles64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
     const int64_t rows128 = (p.M + 127) / 128;
     const int64_t tiles128 = small_tiles <= 64 ? rows128 * ((p.N + 31) / 32) : small_tiles <= 128 ? rows128 * ((p.N + 63) / 64) : small_tiles;
