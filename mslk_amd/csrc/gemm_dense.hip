@@ -200,8 +200,8 @@ bool dense_tiled_supports(const GemmProblem& p) {
 
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (!dense_tiled_supports(p)) return hipErrorInvalidValue;
-  // 256 x 256 tiles once they give every CU work (one persistent workgroup per CU when there are more tiles than
-  // CUs); 128 x 128 below that.
+  // 256 x 256 tiles once they give most CUs work (one persistent workgroup per CU when there are more tiles than
+  // CUs); smaller tiles below that.
   const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
   // 128 x 128 tiles: with at most one tile per CU a workgroup gets the whole LDS for a five-deep ring (its step is
   // much shorter than a memory round trip); with more tiles two workgroups per CU hide each other's latency better.
@@ -226,7 +226,14 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
     if (p.M <= 32 || p.N < 16384) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false>(p, s);
   }
   if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, persistent_workgroups(), s);
-  if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  if (big_tiles >= 160) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  // Between the two: 128 x 256 tiles (wave tile 64 x 128, three ring buffers, one workgroup per CU) when they cover
+  // 160 ... 256 CUs -- fewer LDS bytes per MFMA than 128 x 128 tiles and half the row granularity of 256 x 256
+  // (N = K = 8192, M = 1024: 66.4 -> 59.7 us; N = K = 4096, M = 2048: 31.6 -> 29.0 us).
+  {
+    const int64_t tiles12 = (int64_t)((p.M + 127) / 128) * ((p.N + 255) / 256);
+    if (tiles12 >= 160 && tiles12 <= kCus) return launch_tiled_shape<TileShape<128, 256, 2, 2, 3>, false>(p, s);
+  }
   // M > 64 with at most one 64 x 64 tile per CU: such tiles (four waves stacked along M, five ring buffers, two
   // workgroups per CU) wherever they cover at least as many CUs as the 128-row tiles below would, in a single pass:
   // rows 65 ... 128 then do not cost a second, half-empty 128-row tile's worth of activation traffic (N = K = 8192,

@@ -312,7 +312,8 @@ def test_seeded_random_shape_sweep():
 @pytest.mark.parametrize("M,N,K", [(65, 8192, 8192), (128, 4096, 4096), (200, 2048, 4096), (256, 1024, 8192), (100, 520, 2064),
                                    (384, 4096, 2048), (128, 1024, 14336), (96, 16384, 2048), (130, 64, 272), (70, 136, 144),
                                    (512, 8192, 1024), (66, 72, 16), (65, 4096, 1024), (96, 8192, 400), (128, 7176, 272),
-                                   (250, 4096, 144), (129, 4104, 2048), (100, 6144, 128)])
+                                   (250, 4096, 144), (129, 4104, 2048), (100, 6144, 128), (1000, 8192, 272), (1536, 4104, 144),
+                                   (2048, 5120, 128)])
 def test_medium_m_shapes_use_narrow_and_ring_tiles(M, N, K):
     """Shapes between the skinny kernel (M <= 64) and a full grid of 256 x 256 tiles: 128 x 32 / 128 x 64 / 128 x 128
     tiles with deep operand rings.  Oracle tolerance, both output types, bias, and the pre-shuffled weights."""
