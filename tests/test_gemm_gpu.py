@@ -332,11 +332,13 @@ def test_medium_m_shapes_use_narrow_and_ring_tiles(M, N, K):
         assert_gemm_close(yp, O.dequant_matmul(xq, wq, xs, ws, bias), f"pre-shuffled {M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(4352, 4352, 256), (4100, 4500, 400), (8192, 2304, 128), (2304, 8200, 48), (5000, 4608, 144)])
+@pytest.mark.parametrize("M,N,K", [(4352, 4352, 256), (4100, 4500, 400), (8192, 2304, 128), (2304, 8200, 48), (5000, 4608, 144),
+                                   (2304, 8192, 128), (4609, 4096, 144), (650, 28672, 64), (2561, 8200, 272)])
 def test_more_tiles_than_compute_units(M, N, K):
     """More than 256 tiles of 256 x 256: one persistent workgroup per CU walks several tiles, fetching the next
     tile's first operands before the epilogue of the current one.  Ragged last rows / columns, K tails, one-step and
-    zero-step K loops, both bias types, both output types and the pre-shuffled weights against the oracle."""
+    zero-step K loops, both bias types, both output types and the pre-shuffled weights against the oracle.  The last
+    four shapes leave a last pass less than half full, whose rows a second launch computes with smaller tiles."""
     assert ((M + 255) // 256) * ((N + 255) // 256) > 256
     g = torch.Generator().manual_seed(M + 7 * N + K)
     xq, wq, xs, ws = _random_problem(M, N, K, g)
