@@ -243,20 +243,30 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // M <= 64 on wide row-major weights (the caller sends M <= 8 to the weight-streaming kernel): the activation rows
   // are re-read by every workgroup, so the tile is only as tall as M needs -- 32 x 32 (two waves) or 64 x 32 tiles with
   // six to eight ring buffers, two workgroups per CU.  Measured against the 128-row tiles and the streaming kernel
-  // at N = 5120 ... 28672.
+  // at N = 5120 ... 57344.  Above N = 8192 the 64 x 32 tiles of 32 < M <= 64 no longer fit one per CU and the CUs that
+  // hold two move twice the activation bytes; 64 x 64 tiles halve the tile count and the activation traffic
+  // (N = 10240, K = 8192, M = 64: 33.3 -> 28.3 us; N = 57344, K = 4096, M = 64: 68.4 -> 55.5 us).
   if (p.M <= 64 && p.N >= kShortTileMinN) {
     if (p.M <= 32 && p.N <= 16384) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false>(p, s);
-    if (p.M <= 32 || p.N < 16384) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false>(p, s);
+    if (p.M <= 32 || p.N <= 8192) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false>(p, s);
+    return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false>(p, s);
   }
   if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, persistent_workgroups(), s);
-  if (big_tiles >= 160) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
-  // Between the two: 128 x 256 tiles (wave tile 64 x 128, three ring buffers, one workgroup per CU) when they cover
-  // 160 ... 256 CUs -- fewer LDS bytes per MFMA than 128 x 128 tiles and half the row granularity of 256 x 256
-  // (N = K = 8192, M = 1024: 66.4 -> 59.7 us; N = K = 4096, M = 2048: 31.6 -> 29.0 us).
+  // 128 x 256 tiles (wave tile 64 x 128, three ring buffers, one workgroup per CU) when they cover 160 ... 256 CUs in
+  // a single pass and the 256 x 256 tiles would cover fewer than 160, or would leave their last row of tiles at most
+  // half full -- fewer LDS bytes per MFMA than 128 x 128 tiles and half the row granularity of 256 x 256
+  // (N = K = 8192, M = 1024: 66.4 -> 59.7 us; N = K = 4096, M = 2048: 31.6 -> 29.0 us; N = 57344, K = 8192, M = 128:
+  // 118.5 -> 108.6 us).
   {
-    const int64_t tiles12 = (int64_t)((p.M + 127) / 128) * ((p.N + 255) / 256);
-    if (tiles12 >= 160 && tiles12 <= kCus) return launch_tiled_shape<TileShape<128, 256, 2, 2, 3>, false>(p, s);
+    const int64_t rows128 = (p.M + 127) / 128;
+    const int64_t tiles12 = rows128 * ((p.N + 255) / 256);
+    if (tiles12 >= 160 && tiles12 <= kCus && (big_tiles < 160 || rows128 % 2 == 1))
+      return launch_tiled_shape<TileShape<128, 256, 2, 2, 3>, false>(p, s);
   }
+  // Otherwise 256 x 256 tiles from 129 tiles on: the 128 x 256 tiles would then need two passes and the co-resident
+  // 128 x 128 tiles more than two per CU (N = 6144, M = 1536: 144 tiles, K = 8192: 100.0 -> 87.1 us, K = 4096:
+  // 48.9 -> 39.5 us).
+  if (big_tiles > 128) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
   // M > 64 with at most one 64 x 64 tile per CU: such tiles (four waves stacked along M, five ring buffers, two
   // workgroups per CU) wherever they cover at least as many CUs as the 128-row tiles below would, in a single pass:
   // rows 65 ... 128 then do not cost a second, half-empty 128-row tile's worth of activation traffic (N = K = 8192,

@@ -313,7 +313,8 @@ def test_seeded_random_shape_sweep():
                                    (384, 4096, 2048), (128, 1024, 14336), (96, 16384, 2048), (130, 64, 272), (70, 136, 144),
                                    (512, 8192, 1024), (66, 72, 16), (65, 4096, 1024), (96, 8192, 400), (128, 7176, 272),
                                    (250, 4096, 144), (129, 4104, 2048), (100, 6144, 128), (1000, 8192, 272), (1536, 4104, 144),
-                                   (2048, 5120, 128)])
+                                   (2048, 5120, 128), (1536, 6144, 144), (1500, 6152, 128), (128, 57344, 128), (100, 50000, 144),
+                                   (384, 20480, 128)])
 def test_medium_m_shapes_use_narrow_and_ring_tiles(M, N, K):
     """Shapes between the skinny kernel (M <= 64) and a full grid of 256 x 256 tiles: 128 x 32 / 128 x 64 / 128 x 128
     tiles with deep operand rings.  Oracle tolerance, both output types, bias, and the pre-shuffled weights."""
@@ -360,10 +361,11 @@ def test_more_tiles_than_compute_units(M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(9, 8192, 1024), (16, 8200, 512), (32, 16384, 384), (24, 20000, 272), (33, 8192, 2048),
                                    (48, 12296, 144), (64, 9000, 1040), (64, 16383, 128), (40, 28672, 256), (17, 8192, 16),
-                                   (12, 5120, 1024), (64, 6152, 400), (31, 7168, 2048)])
+                                   (12, 5120, 1024), (64, 6152, 400), (31, 7168, 2048), (48, 9216, 272), (64, 20488, 144),
+                                   (33, 57344, 128), (64, 8200, 1024)])
 def test_small_m_on_wide_weights_uses_short_tiles(M, N, K):
-    """8 < M <= 64 with N >= 5120 and row-major weights: 32 x 32 and 64 x 32 tiles (two- and four-wave workgroups, deep
-    operand rings) instead of the weight-streaming kernel.  Ragged rows and columns, K tails, bias, fp16 output."""
+    """8 < M <= 64 with N >= 5120 and row-major weights: 32 x 32, 64 x 32 and (32 < M, N > 8192) 64 x 64 tiles (two- and
+    four-wave workgroups, deep operand rings) instead of the weight-streaming kernel.  Ragged rows and columns, K tails, bias, fp16 output."""
     g = torch.Generator().manual_seed(M * 5 + N + K)
     xq, wq, xs, ws = _random_problem(M, N, K, g)
     bias = (torch.randn(N, generator=g) * 0.5).float()
