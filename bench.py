@@ -157,6 +157,50 @@ def cpu_baseline(wl, budget_s=20.0):
                       f"N={N}, K={K}, median of 3, {t * 1e3:.1f} ms; os.cpu_count()={os.cpu_count()}"}
 
 
+def _vendor_sweep(api):
+    """`--only vendor`: this library against the vendor library (hipBLASLt behind torch._scaled_mm, row-wise scales) on
+    weight shapes of 8B / 70B-class models at M = 1 ... 16384; same operands, rotating sets larger than the caches,
+    best of three event-timed loops.  Prints one line per shape and a summary line (JSON)."""
+    import torch
+    import mslk_amd
+    dev = "cuda:0"
+    ratios = []
+    for (N, K) in [(8192, 8192), (10240, 8192), (57344, 8192), (8192, 28672), (4096, 4096), (6144, 4096), (28672, 4096), (4096, 14336)]:
+        nsets = 6 if N * K < 2 ** 27 else 3
+        g = torch.Generator(device=dev).manual_seed(N + K)
+        weights = [mslk_amd.quantize_fp8_row(torch.randn(N, K, device=dev, generator=g).bfloat16()) for _ in range(nsets)]
+        for M in (1, 16, 64, 128, 256, 384, 512, 1024, 2048, 4096, 8192, 16384):
+            acts = [mslk_amd.quantize_fp8_row(torch.randn(M, K, device=dev, generator=g).bfloat16()) for _ in range(nsets)]
+            ys = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nsets)]
+
+            def ours(i):
+                j = i % nsets
+                api.gemm(acts[j][0], weights[j][0], acts[j][1], weights[j][1], ys[j])
+
+            def vendor(i):
+                j = i % nsets
+                torch._scaled_mm(acts[j][0], weights[j][0].t(), scale_a=acts[j][1][:, None], scale_b=weights[j][1][None, :],
+                                 out_dtype=torch.bfloat16)
+
+            def best_us(fn):
+                for i in range(8):
+                    fn(i)
+                torch.cuda.synchronize()
+                return min(_events_ms(fn, 40) for _ in range(3)) * 1e3
+
+            vendor(0)   # the first call picks the vendor kernel
+            t_vendor, t_ours = best_us(vendor), best_us(ours)
+            ratios.append(t_vendor / t_ours)
+            print(f"M={M:6d} N={N:6d} K={K:6d}: ours {t_ours:8.1f} us {2.0 * M * N * K / t_ours / 1e9:5.2f} PFLOP/s | "
+                  f"vendor {t_vendor:8.1f} us | vendor/ours {t_vendor / t_ours:4.2f}", flush=True)
+            del acts, ys
+        del weights
+        torch.cuda.empty_cache()
+    ratios.sort()
+    print(json.dumps({"shapes": len(ratios), "ours_faster": sum(r > 1.0 for r in ratios), "median_ratio": round(ratios[len(ratios) // 2], 3),
+                      "min_ratio": round(ratios[0], 3), "max_ratio": round(ratios[-1], 3)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -164,7 +208,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", default="", help="profile helper: run only this piece (gemm|quantize|decode|traffic) and exit")
+    ap.add_argument("--only", default="", help="helper: run only this piece (gemm|quantize|decode|traffic|vendor) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -179,6 +223,9 @@ def main():
     torch.cuda.set_device(dev)
     api = CApi()
     extras = {}
+    if args.only == "vendor":
+        _vendor_sweep(api)
+        return
 
     # ---------------------------------------------------------------- cfg1: 4096^3
     wl = W.cfg1()
