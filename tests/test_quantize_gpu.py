@@ -76,6 +76,33 @@ def test_reference_shape_sweep(dtype):
         assert_quant_bit_exact(a, xq, s)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_many_short_rows(dtype):
+    """4096 rows and more of K <= 256 (per-head quantization): 8 / 16 / 32 lanes per row, several rows per wavefront.
+    Ragged row counts, K on both sides of each team width, scale_ub, padded output rows, a jagged batch."""
+    g = torch.Generator().manual_seed(12)
+    for rows, K in [(4096, 8), (4099, 64), (5000, 72), (4097, 128), (6001, 136), (4100, 256), (4096, 16), (8200, 120),
+                    (4101, 200), (4096, 264)]:
+        a = (torch.randn(rows, K, generator=g) * torch.logspace(-3, 3, rows)[:, None]).to(dtype)
+        a[7] = 0
+        xq, s = _run(a)
+        assert_quant_bit_exact(a, xq, s)
+    a = (torch.randn(4500, 128, generator=g) * 3).to(dtype)
+    t = torch.tensor([1.5], dtype=torch.float32)
+    xq, s = _run(a, scale_ub=t)
+    assert_quant_bit_exact(a, xq, s, scale_ub=t)
+    a = torch.randn(4200, 100 if dtype != torch.float32 else 104, generator=g).to(dtype)
+    if a.shape[1] % 8 == 0:
+        xq, s = _run(a, align=16)
+        assert_quant_bit_exact(a, xq, s, K_out=112)
+    b = torch.randn(8, 600, 128, generator=g).to(dtype)          # 4800 rows in 8 groups, some rows dead
+    zs = torch.tensor([600, 0, 1, 599, 300, 17, 600, 64], dtype=torch.int64)
+    xq, s = mslk_amd.quantize_fp8_row(b.to(DEV), zero_start_index_M=zs.to(DEV))
+    torch.cuda.synchronize()
+    rq, rs = O.quantize_fp8_row_jagged(b, zs)
+    assert torch.equal(codes(xq), codes(rq)) and torch.equal(bits32(s), bits32(rs))
+
+
 def test_special_rows_and_magnitudes():
     g = torch.Generator().manual_seed(3)
     a = (torch.randn(512, 2048, generator=g) * torch.logspace(-20, 20, 512)[:, None]).to(torch.bfloat16)
