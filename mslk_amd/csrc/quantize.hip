@@ -353,6 +353,9 @@ hipError_t launch_quantize_t(const void* x, int64_t rows, int64_t K, int64_t in_
     quantize_rows_vec_kernel<DTYPE, 256, 4, true, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else if (K <= 256 * 8 * NV) {
     quantize_rows_vec_kernel<DTYPE, 256, NV, true, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
+  } else if (DTYPE != 2 && K <= 256 * 8 * 32) {
+    // 16-bit rows up to 65536 elements still fit the registers of one workgroup (32 x 16 bytes per lane)
+    quantize_rows_vec_kernel<DTYPE, 256, (DTYPE != 2 ? 32 : 1), true, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   } else {
     quantize_rows_vec_kernel<DTYPE, 256, 1, false, TRITON><<<(unsigned)rows, 256, 0, s>>>(x, rows, k, in_stride, out, out_stride, scale, scale_ub, jag);
   }

@@ -69,7 +69,8 @@ def test_reference_shape_sweep(dtype):
     g = torch.Generator().manual_seed(2)
     shapes = [(2, n) for n in range(1, 9000, 100)]
     shapes += [(16, 16), (64, 512), (1024, 1024), (4096, 2048), (8192, 4096), (333, 777), (1, 128), (128, 1),
-               (5, 8192), (3, 16384), (2, 40000), (2, 70008), (2500, 8192), (64, 8192), (1, 8192)]
+               (5, 8192), (3, 16384), (2, 40000), (2, 70008), (2500, 8192), (64, 8192), (1, 8192), (5, 65536), (3, 57344),
+               (2, 32776), (2, 65544)]
     for shape in shapes:
         a = torch.randn(shape, generator=g).to(dtype)
         xq, s = _run(a)
