@@ -300,6 +300,27 @@ __global__ __launch_bounds__(256) void dequantize_rows_vec_kernel(const uint8_t*
   }
 }
 
+// As above for K % 8 == 0 (rows of codes 8-byte aligned, rows of the output 16-byte aligned): 8 codes per lane.
+__global__ __launch_bounds__(256) void dequantize_rows_vec8_kernel(const uint8_t* __restrict__ xq,
+                                                                   const float* __restrict__ scale, int64_t chunks,
+                                                                   int chunks_per_row, uint16_t* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += stride) {
+    const v2i q = __builtin_nontemporal_load(reinterpret_cast<const v2i*>(xq) + c);
+    const float sc = scale[c / chunks_per_row];
+    const int w[2] = {q.x, q.y};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(w[i], false);
+      const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(w[i], true);
+      o[2 * i] = pack_bf16x2(lo[0] * sc, lo[1] * sc);
+      o[2 * i + 1] = pack_bf16x2(hi[0] * sc, hi[1] * sc);
+    }
+    __builtin_nontemporal_store(v4i{(int)o[0], (int)o[1], (int)o[2], (int)o[3]}, reinterpret_cast<v4i*>(out) + c);
+  }
+}
+
 __global__ __launch_bounds__(256) void dequantize_rows_generic_kernel(const uint8_t* __restrict__ xq,
                                                                       const float* __restrict__ scale, int64_t total,
                                                                       int64_t K, uint16_t* __restrict__ out) {
@@ -396,6 +417,12 @@ hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t
     const unsigned blocks = (unsigned)(want > 256 * 32 ? 256 * 32 : want);
     dequantize_rows_vec_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const uint8_t*>(xq), scale, chunks, (int)(K / 16),
                                                      reinterpret_cast<uint16_t*>(out));
+  } else if (K % 8 == 0 && reinterpret_cast<uintptr_t>(xq) % 8 == 0 && reinterpret_cast<uintptr_t>(out) % 16 == 0) {
+    const int64_t chunks = total / 8;
+    const int64_t want = (chunks + 255) / 256;
+    const unsigned blocks = (unsigned)(want > 256 * 32 ? 256 * 32 : want);
+    dequantize_rows_vec8_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const uint8_t*>(xq), scale, chunks, (int)(K / 8),
+                                                      reinterpret_cast<uint16_t*>(out));
   } else {
     const int64_t want = (total + 255) / 256;
     const unsigned blocks = (unsigned)(want > 65536 ? 65536 : want);

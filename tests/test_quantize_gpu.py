@@ -215,7 +215,8 @@ def test_jagged_rows(shape, align, idx_dtype):
     assert s.shape == a.shape[:-1]
 
 
-@pytest.mark.parametrize("shape", [(1, 256), (3, 16), (7, 777), (64, 1024), (2, 3, 17, 136), (2500, 4096), (5, 3)])
+@pytest.mark.parametrize("shape", [(1, 256), (3, 16), (7, 777), (64, 1024), (2, 3, 17, 136), (2500, 4096), (5, 3), (300, 4104),
+                                   (4096, 520), (33, 8), (1000, 1000)])
 def test_dequantize_bit_exact(shape):
     g = torch.Generator().manual_seed(sum(shape))
     rows = 1
