@@ -190,31 +190,36 @@ def ck_preshuffle(src: torch.Tensor, NXdl: int = 16) -> torch.Tensor:
 
 
 def _check_grouped(XQ: Sequence[torch.Tensor], WQ, x_scale, w_scale):
-    _check(len(XQ) == len(WQ) == len(x_scale) == len(w_scale), "All inputs must have the same number of groups.")
-    for x in XQ:
-        _check(x.is_cuda and x.is_contiguous(), "XQ tensors must be contiguous GPU tensors")
-        _check(x.dim() == 2, "Inputs must be 2D.")
-    for w in WQ:
-        _check(w.is_cuda and w.is_contiguous(), "WQ tensors must be contiguous GPU tensors")
-        _check(w.dim() == 2, "Inputs must be 2D.")
-        _check(XQ[0].dtype == w.dtype, f"XQ and WQ dtypes must match, got {XQ[0].dtype} vs {w.dtype}")
-        _check(w.shape[0] >= 512 and w.shape[1] >= 512,
-               "N and K must be at least 512 for grouped gemm. For smaller inputs, consider unrolling.")
-    for s in list(x_scale) + list(w_scale):
-        _check(s.dtype == torch.float32, "Scales must be float32.")
-    if len(XQ):
-        _check(XQ[0].dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ[0].dtype}")
+    """Argument checks of the TensorList ops; one pass over the groups (this runs on every call of a decode loop, so the
+    common case costs a few comparisons per group and messages are only built on failure)."""
+    G = len(XQ)
+    _check(G == len(WQ) == len(x_scale) == len(w_scale), "All inputs must have the same number of groups.")
+    if G == 0:
+        return
+    dev, f32 = XQ[0].device, torch.float32
+    _check(XQ[0].dtype == FP8_DTYPE, f"XQ and WQ must be {FP8_DTYPE} on gfx950, got {XQ[0].dtype}")
     for x, w, xs, ws in zip(XQ, WQ, x_scale, w_scale):
-        _check(x.shape[1] == w.shape[1], "XQ and WQ of a group must share K")
-        _check(xs.numel() == x.shape[0] and ws.numel() == w.shape[0], "scale sizes must match M and N of their group")
-        _check(w.device == x.device and xs.device == x.device and ws.device == x.device and x.device == XQ[0].device,
+        xsh, wsh = x.shape, w.shape
+        if not (x.is_cuda and w.is_cuda and x.is_contiguous() and w.is_contiguous()):
+            _check(x.is_cuda and x.is_contiguous(), "XQ tensors must be contiguous GPU tensors")
+            _check(False, "WQ tensors must be contiguous GPU tensors")
+        _check(len(xsh) == 2 and len(wsh) == 2, "Inputs must be 2D.")
+        if w.dtype != FP8_DTYPE or x.dtype != FP8_DTYPE:
+            other = w.dtype if w.dtype != FP8_DTYPE else x.dtype
+            _check(False, f"XQ and WQ dtypes must match, got {FP8_DTYPE} vs {other}")
+        _check(wsh[0] >= 512 and wsh[1] >= 512,
+               "N and K must be at least 512 for grouped gemm. For smaller inputs, consider unrolling.")
+        _check(xs.dtype == f32 and ws.dtype == f32, "Scales must be float32.")
+        _check(xsh[1] == wsh[1], "XQ and WQ of a group must share K")
+        _check(xs.numel() == xsh[0] and ws.numel() == wsh[0], "scale sizes must match M and N of their group")
+        _check(x.device == dev and w.device == dev and xs.device == dev and ws.device == dev,
                "all operands must be on the same device")
 
 
 def _launch_grouped(XQ, WQ, x_scale, w_scale, outs: List[torch.Tensor]) -> None:
     G = len(XQ)
-    xs = [s.contiguous() for s in x_scale]
-    ws = [s.contiguous() for s in w_scale]
+    xs = [s if s.is_contiguous() else s.contiguous() for s in x_scale]
+    ws = [s if s.is_contiguous() else s.contiguous() for s in w_scale]
     PtrArr = ctypes.c_void_p * G
     I64Arr = ctypes.c_int64 * G
     dev = XQ[0].device
@@ -233,9 +238,14 @@ def f8f8bf16_rowwise_grouped(XQ, WQ, x_scale, w_scale) -> List[torch.Tensor]:
     _check_grouped(XQ, WQ, x_scale, w_scale)
     if len(XQ) == 0:
         return []
-    sizes = [x.shape[0] * w.shape[0] for x, w in zip(XQ, WQ)]
-    flat = torch.empty(sum(sizes), dtype=torch.bfloat16, device=XQ[0].device)
-    outs = [t.view(x.shape[0], w.shape[0]) for t, x, w in zip(flat.split(sizes), XQ, WQ)]
+    Ms = [x.shape[0] for x in XQ]
+    Ns = [w.shape[0] for w in WQ]
+    if Ns.count(Ns[0]) == len(Ns):   # one N: the row blocks of a [sum M, N] buffer are the same views, made by one call
+        outs = list(torch.empty((sum(Ms), Ns[0]), dtype=torch.bfloat16, device=XQ[0].device).split(Ms))
+    else:
+        sizes = [m * n for m, n in zip(Ms, Ns)]
+        flat = torch.empty(sum(sizes), dtype=torch.bfloat16, device=XQ[0].device)
+        outs = [t.view(m, n) for t, m, n in zip(flat.split(sizes), Ms, Ns)]
     _launch_grouped(XQ, WQ, x_scale, w_scale, outs)
     return outs
 
