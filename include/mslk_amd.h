@@ -130,8 +130,13 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
  * math csrc/gemm/ck/fp8_rowwise/kernels/fp8_rowwise_common.h:54-82,168-204; bias semantics
  * csrc/gemm/cutlass/f8f8bf16_rowwise/f8f8bf16_rowwise_common.cuh:150-198).
  * M, N or K equal to 0 writes zeros to Y (fp8fp8bf16_rowwise_gemm.hip:531-534).
- * `workspace` is only needed when mslk_amd_f8f8bf16_rowwise_workspace_bytes(M,N,K) > 0; it must be
- * zero-filled before its first use and is left zero-filled by every call (split-K arrival counters).
+ * `workspace` (device memory, 16-byte aligned) is optional and only used when
+ * mslk_amd_f8f8bf16_rowwise_workspace_bytes(M,N,K) > 0, i.e. when K is not a multiple of 16: the call then copies both
+ * operands into workspace rows of K rounded up to 16 (zero tail) and runs the MFMA kernels on the copies (the CK
+ * instances of the reference pad K inside the kernel, fp8_rowwise_common.h:109-110 `GemmSpecialization::MNKPadding`).
+ * Without a workspace (null or too small) such a K still gives the same results through a scalar kernel that is
+ * orders of magnitude slower.  The workspace needs no initialisation and holds nothing between calls; calls that
+ * share one workspace must not overlap.
  */
 int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                               const void* bias, int bias_dtype, void* y,
@@ -142,11 +147,11 @@ size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K
 /*
  * The same GEMM with an fp16 (IEEE half, round to nearest even, overflow to infinity) output.
  * Replaces mslk::gemm::f8f8f16_rowwise (reference: csrc/gemm/gemm_ops.cpp:88-89,
- * csrc/gemm/ck/fp8_rowwise/fp8fp8fp16_rowwise_gemm.hip:66-133).  Arguments as above; y is fp16.
+ * csrc/gemm/ck/fp8_rowwise/fp8fp8fp16_rowwise_gemm.hip:66-133).  Arguments as above (the same workspace rule); y is fp16.
  */
 int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
-                             void* stream);
+                             void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * The dense GEMM on PRE-SHUFFLED weights.  Replaces mslk::gemm::f8f8bf16_rowwise_preshuffle and

@@ -33,7 +33,7 @@ SIGNATURES = {
     "mslk_amd_f8f8bf16_rowwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                           c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "mslk_amd_f8f8f16_rowwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
-                                         c_int64, c_int64, c_int64, c_void_p]),
+                                         c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "mslk_amd_f8f8_rowwise_preshuffle": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                                  c_int64, c_int64, c_int64, c_void_p]),
     "mslk_amd_preshuffle_b": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),

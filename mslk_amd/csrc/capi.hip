@@ -144,11 +144,17 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
   return check_hip(launch_fused_quant(p, kFusedGatherScale, (hipStream_t)stream), "gather_scale_quant launch");
 }
 
-size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t, int64_t, int64_t) { return 0; }
+// K that is not a multiple of 16: the operand rows cannot be fetched by the 16-byte loads of the MFMA kernels.  With a
+// workspace the call copies both operands into rows of K rounded up to 16 (zero tail: code 0x00 is +0) and runs the
+// ordinary kernels on the copies; without one it falls back to the scalar kernel, which is orders of magnitude slower.
+size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % 16 == 0) return 0;
+  return (size_t)((M + N) * ((K + 15) / 16 * 16));
+}
 
 static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void* xq, const void* wq, const float* x_scale,
                         const float* w_scale, const void* bias, int bias_dtype, void* y, int64_t M, int64_t N,
-                        int64_t K, void* stream) {
+                        int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
   if (M < 0 || N < 0 || K < 0) return fail("%s: negative dimension", op);
   if (M > kIntMax || N > kIntMax || K > kIntMax) return fail("%s: dimension exceeds 2^31-1", op);
   if (bias_dtype < 0 || bias_dtype > 2) return fail("%s: bad bias dtype code %d", op, bias_dtype);
@@ -162,6 +168,20 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
     return fail("%s: pre-shuffled weights need N %% 16 == 0 and K %% 64 == 0 (got N=%lld, K=%lld)", op, (long long)N, (long long)K);
   GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
                 (int)M, (int)N, (int)K, bias_dtype, out_f16, preshuffled};
+  const size_t pad_bytes = mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K);
+  if (pad_bytes > 0 && !preshuffled && workspace && workspace_bytes >= pad_bytes &&
+      reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+    const int64_t Kp = (K + 15) / 16 * 16;
+    if (Kp <= kIntMax) {
+      uint8_t* xp = static_cast<uint8_t*>(workspace);
+      uint8_t* wp = xp + M * Kp;
+      if (int rc = check_hip(launch_pad_rows(p.xq, xp, M, K, Kp, s), "pad rows launch")) return rc;
+      if (int rc = check_hip(launch_pad_rows(p.wq, wp, N, K, Kp, s), "pad rows launch")) return rc;
+      p.xq = xp;
+      p.wq = wp;
+      p.K = (int)Kp;
+    }
+  }
   // M <= 64: the weight-streaming kernel, except on wide row-major weights, where short tiles that share their
   // activation rows through LDS win from M = 9 on.  Pre-shuffled weights
   // keep the streaming kernel, whose register-direct weight loads stay ahead up to M = 64.
@@ -174,14 +194,14 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
 
 int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                               const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
-                              void* /*workspace*/, size_t /*workspace_bytes*/, void* stream) {
-  return rowwise_impl("f8f8bf16_rowwise", 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  return rowwise_impl("f8f8bf16_rowwise", 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, workspace, workspace_bytes, stream);
 }
 
 int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
-                             void* stream) {
-  return rowwise_impl("f8f8f16_rowwise", 1, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+                             void* workspace, size_t workspace_bytes, void* stream) {
+  return rowwise_impl("f8f8f16_rowwise", 1, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, workspace, workspace_bytes, stream);
 }
 
 int mslk_amd_f8f8_rowwise_preshuffle(const void* xq, const void* wq_shuffled, const float* x_scale, const float* w_scale,
@@ -190,7 +210,7 @@ int mslk_amd_f8f8_rowwise_preshuffle(const void* xq, const void* wq_shuffled, co
   if (y_dtype != MSLK_AMD_DTYPE_BF16 && y_dtype != MSLK_AMD_DTYPE_F16)
     return fail("f8f8_rowwise_preshuffle: output dtype code %d is neither bf16 nor fp16", y_dtype);
   return rowwise_impl(y_dtype == MSLK_AMD_DTYPE_F16 ? "f8f8f16_rowwise_preshuffle" : "f8f8bf16_rowwise_preshuffle",
-                      y_dtype == MSLK_AMD_DTYPE_F16, 1, xq, wq_shuffled, x_scale, w_scale, bias, bias_dtype, y, M, N, K, stream);
+                      y_dtype == MSLK_AMD_DTYPE_F16, 1, xq, wq_shuffled, x_scale, w_scale, bias, bias_dtype, y, M, N, K, nullptr, 0, stream);
 }
 
 int mslk_amd_preshuffle_b(const void* wq, void* wq_shuffled, int64_t G, int64_t N, int64_t K, void* stream) {

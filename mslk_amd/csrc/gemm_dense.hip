@@ -184,6 +184,27 @@ __global__ __launch_bounds__(256) void preshuffle_b_kernel(const v4i* __restrict
   }
 }
 
+// Rows of K bytes copied into rows of Kp bytes with a zero tail: one lane per 16-byte chunk of the destination.
+// The source rows start at any byte, so the reads carry no alignment promise.
+__global__ __launch_bounds__(256) void pad_rows_kernel(const uint8_t* __restrict__ src, uint8_t* __restrict__ dst,
+                                                       int64_t chunks, int chunks_per_row, int K) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += stride) {
+    const int64_t row = c / chunks_per_row;
+    const int k0 = (int)(c - row * chunks_per_row) * 16;
+    const uint8_t* in = src + row * K + k0;
+    uint32_t w[4] = {0u, 0u, 0u, 0u};
+    if (k0 + 16 <= K) {
+      __builtin_memcpy(w, in, 16);   // alignment 1: the compiler picks whatever access width the target allows
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        if (k0 + i < K) w[i >> 2] |= (uint32_t)in[i] << (8 * (i & 3));
+    }
+    reinterpret_cast<v4i*>(dst)[c] = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+  }
+}
+
 __global__ void fill_zero_kernel(uint16_t* y, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) y[i] = 0;
@@ -295,6 +316,14 @@ hipError_t launch_preshuffle_b(const void* src, void* dst, int64_t G, int64_t N,
   const int64_t want = (chunks + 255) / 256;
   preshuffle_b_kernel<<<(unsigned)(want > 65536 ? 65536 : want), 256, 0, s>>>(static_cast<const v4i*>(src), static_cast<v4i*>(dst),
                                                                               chunks, (int)K);
+  return hipGetLastError();
+}
+
+hipError_t launch_pad_rows(const uint8_t* src, uint8_t* dst, int64_t rows, int64_t K, int64_t Kp, hipStream_t s) {
+  const int64_t chunks = rows * (Kp / 16);
+  if (chunks <= 0) return hipSuccess;
+  const int64_t want = (chunks + 255) / 256;
+  pad_rows_kernel<<<(unsigned)(want > 65536 ? 65536 : want), 256, 0, s>>>(src, dst, chunks, (int)(Kp / 16), (int)K);
   return hipGetLastError();
 }
 

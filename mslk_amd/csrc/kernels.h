@@ -67,6 +67,8 @@ constexpr int kShortTileMinN = 5120;
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s);
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s);   // any shape, slow
 hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s);
+// dst[r, 0:K] = src[r, 0:K], dst[r, K:Kp] = 0 for `rows` rows of bytes (Kp a multiple of 16, dst 16-byte aligned)
+hipError_t launch_pad_rows(const uint8_t* src, uint8_t* dst, int64_t rows, int64_t K, int64_t Kp, hipStream_t s);
 
 // Grouped problems.  Up to kMaxGroupsPerLaunch descriptors travel in the kernel argument block.
 constexpr int kMaxGroupsPerLaunch = 64;

@@ -128,15 +128,17 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, o
                 XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
                 1 if out_dtype == torch.float16 else 0, M, N, K, _stream_ptr(XQ.device)))
         return Y
+    wsp_ptr, wsp_bytes = None, 0
+    if K % 16:
+        # rows the 16-byte loads cannot fetch: room for copies with K rounded up (the caching allocator's block, so the
+        # call stays capturable); the library pads into it and runs the MFMA kernels on the copies
+        wsp_bytes = (M + N) * ((K + 15) // 16 * 16)
+        wsp = torch.empty(wsp_bytes, dtype=torch.uint8, device=XQ.device)
+        wsp_ptr = wsp.data_ptr()
     with _on_device(XQ.device):
-        if out_dtype == torch.float16:
-            _lib.check(_lib.lib().mslk_amd_f8f8f16_rowwise(
-                XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
-                M, N, K, _stream_ptr(XQ.device)))
-        else:
-            _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise(
-                XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
-                M, N, K, None, 0, _stream_ptr(XQ.device)))
+        fn = _lib.lib().mslk_amd_f8f8f16_rowwise if out_dtype == torch.float16 else _lib.lib().mslk_amd_f8f8bf16_rowwise
+        _lib.check(fn(XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
+                      M, N, K, wsp_ptr, wsp_bytes, _stream_ptr(XQ.device)))
     return Y
 
 

@@ -140,6 +140,44 @@ def test_unaligned_views_take_the_generic_path():
     assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws))
 
 
+@pytest.mark.parametrize("M,N,K", [(300, 520, 1000), (1, 8192, 8200), (16, 8192, 8190), (64, 600, 17), (5, 7, 1), (512, 4096, 1001),
+                                   (1030, 2050, 4100), (40, 5200, 2047), (700, 300, 15)])
+def test_k_not_a_multiple_of_16_runs_on_padded_copies(M, N, K):
+    """K % 16 != 0: the ops hand the library a workspace, it copies both operands into rows of K rounded up to 16
+    (zero tail) and runs the MFMA kernels on the copies.  Same tolerance as every other shape, with bias, both output
+    types; through the C ABI the result without a workspace (scalar kernel) has to agree as well, and the reported
+    workspace size is the documented one."""
+    from mslk_amd import _lib
+    g = torch.Generator().manual_seed(M + 3 * N + 5 * K)
+    xq, wq, xs, ws = _random_problem(M, N, K, g)
+    bias = (torch.randn(N, generator=g) * 0.5).float()
+    d = _gpu(xq, wq, xs, ws)
+    y = torch.ops.mslk.f8f8bf16_rowwise(*d, bias=bias.to(DEV))
+    y16 = torch.ops.mslk.f8f8f16_rowwise(*d)
+    out = torch.full((M, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+    torch.ops.mslk.f8f8bf16_rowwise_out(*d, out)
+    torch.cuda.synchronize()
+    ref = O.dequant_matmul(xq, wq, xs, ws)
+    assert_gemm_close(y, ref + bias, f"{M}x{N}x{K}")
+    assert_gemm_close(y16, ref, f"fp16 {M}x{N}x{K}")
+    assert_gemm_close(out, ref, f"out {M}x{N}x{K}")
+    L = _lib.lib()
+    Kp = (K + 15) // 16 * 16
+    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K) == (M + N) * Kp
+    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, Kp) == 0
+    if M * N * K <= 2 ** 31:   # the scalar kernel is slow
+        y_plain = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        _lib.check(L.mslk_amd_f8f8bf16_rowwise(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), None, 0,
+                                               y_plain.data_ptr(), M, N, K, None, 0, None))
+        small = torch.empty(16, dtype=torch.uint8, device=DEV)   # a workspace that is too small is ignored
+        y_small = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        _lib.check(L.mslk_amd_f8f8bf16_rowwise(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), None, 0,
+                                               y_small.data_ptr(), M, N, K, small.data_ptr(), 16, None))
+        torch.cuda.synchronize()
+        assert_gemm_close(y_plain, ref, f"no workspace {M}x{N}x{K}")
+        assert torch.equal(y_plain.view(torch.int16), y_small.view(torch.int16))
+
+
 @pytest.mark.parametrize("M,N,K", [(512, 1024, 512), (16, 1024, 1024), (4352, 4352, 128), (16, 8192, 256), (64, 8192, 256)])
 def test_hip_graph_capture_and_replay(M, N, K):
     """The reference tests capture + replay (test/gemm/gemm_test.py:440-447); replay several times with
