@@ -615,6 +615,10 @@ struct GemmTile {
           if (mm >= m_rem || nn >= n_rem) continue;
           if (vec_store && nn + 7 < n_rem) {
             store16_stream(dst, val);
+          } else if (nn + 7 < n_rem) {
+            // all eight columns valid, but rows of Y are only 2- or 4-byte aligned (N % 8 != 0): a 16-byte copy with
+            // no alignment promise, for which the compiler picks the widest store the target allows
+            __builtin_memcpy(dst, &val, 16);
           } else if (pair_store) {   // rows are 4-byte aligned: store bf16 pairs
             const uint32_t w[4] = {val.x, val.y, val.z, val.w};
             uint32_t* d32 = reinterpret_cast<uint32_t*>(dst);
