@@ -242,7 +242,9 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
   for (int64_t k = K + lane; k < out_stride; k += TEAM) out[row * out_stride + k] = 0;
 }
 
-// Generic path: any K, any alignment; one workgroup per row, scalar accesses, two passes.
+// Generic path: any K, any alignment; one workgroup per row, two passes.  Full groups of eight elements move as 16- / 32-byte
+// copies without an alignment promise (the compiler picks the access width the target allows), the K % 8 tail and the
+// padding columns element by element.
 template <int DTYPE, bool TRITON>
 __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
     const void* __restrict__ x, int64_t rows, int64_t K, int64_t in_stride, uint8_t* __restrict__ out,
@@ -252,8 +254,16 @@ __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
   const int64_t row = blockIdx.x;
   const elem_t* xr = reinterpret_cast<const elem_t*>(x) + row * in_stride;
   if (!row_is_live(jag, row)) K = 0;   // nothing of the row is read; all codes become zero
+  const int64_t nvec = K >> 3;
+  const char* xb = reinterpret_cast<const char*>(xr);
   uint32_t m = 0;
-  for (int64_t k = threadIdx.x; k < K; k += 256) {
+  for (int64_t idx = threadIdx.x; idx < nvec; idx += 256) {
+    Vec8<DTYPE> v;
+    __builtin_memcpy(&v, xb + idx * sizeof(Vec8<DTYPE>), sizeof(Vec8<DTYPE>));
+    m = absmax_bits<DTYPE>(m, v);
+  }
+  m = finish_absmax_bits<DTYPE>(m);
+  for (int64_t k = nvec * 8 + threadIdx.x; k < K; k += 256) {
     if constexpr (DTYPE == 2) m = max(m, __float_as_uint(xr[k]) & 0x7FFFFFFFu);
     else m = max(m, (uint32_t)xr[k] & 0x7FFFu);
   }
@@ -261,7 +271,14 @@ __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
   float inv, sc;
   scales_from_amax<DTYPE, TRITON>(Traits<DTYPE>::abs_bits_to_f32(m), scale_ub, jag.triton_eps, inv, sc);
   if (threadIdx.x == 0) scale[row] = sc;
-  for (int64_t k = threadIdx.x; k < out_stride; k += 256) {
+  uint8_t* out_row = out + row * out_stride;
+  for (int64_t idx = threadIdx.x; idx < nvec; idx += 256) {
+    Vec8<DTYPE> v;
+    __builtin_memcpy(&v, xb + idx * sizeof(Vec8<DTYPE>), sizeof(Vec8<DTYPE>));
+    const uint2 q = quantize_vec8<DTYPE, TRITON>(v, inv);
+    __builtin_memcpy(out_row + idx * 8, &q, 8);
+  }
+  for (int64_t k = nvec * 8 + threadIdx.x; k < out_stride; k += 256) {
     uint8_t code = 0;
     if (k < K) {
       float f;
@@ -271,7 +288,7 @@ __global__ __launch_bounds__(256) void quantize_rows_generic_kernel(
       else f = f * inv;
       code = (uint8_t)(cvt_pk_e4m3fn(f, 0.0f) & 0xFFu);
     }
-    out[row * out_stride + k] = code;
+    out_row[k] = code;
   }
 }
 
@@ -321,12 +338,35 @@ __global__ __launch_bounds__(256) void dequantize_rows_vec8_kernel(const uint8_t
   }
 }
 
+// Any K, any alignment: a lane takes 8 consecutive codes of the flat tensor; when they lie in one row they move as an
+// 8-byte and a 16-byte copy without an alignment promise, otherwise (row boundary, end of the tensor) one by one.
 __global__ __launch_bounds__(256) void dequantize_rows_generic_kernel(const uint8_t* __restrict__ xq,
                                                                       const float* __restrict__ scale, int64_t total,
                                                                       int64_t K, uint16_t* __restrict__ out) {
   const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
-    out[i] = (uint16_t)f32_to_bf16_bits(__builtin_amdgcn_cvt_f32_fp8((int)xq[i], 0) * scale[i / K]);
+  const int64_t chunks = (total + 7) / 8;
+  for (int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x; c < chunks; c += stride) {
+    const int64_t i0 = c * 8;
+    const int n = total - i0 < 8 ? (int)(total - i0) : 8;
+    const int64_t r0 = i0 / K;
+    if (n == 8 && (i0 + 7) / K == r0) {
+      uint32_t w[2];
+      __builtin_memcpy(w, xq + i0, 8);
+      const float sc = scale[r0];
+      uint32_t o[4];
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], false);
+        const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)w[i], true);
+        o[2 * i] = pack_bf16x2(lo[0] * sc, lo[1] * sc);
+        o[2 * i + 1] = pack_bf16x2(hi[0] * sc, hi[1] * sc);
+      }
+      __builtin_memcpy(out + i0, o, 16);
+    } else {
+      for (int e = 0; e < n; ++e)
+        out[i0 + e] = (uint16_t)f32_to_bf16_bits(__builtin_amdgcn_cvt_f32_fp8((int)xq[i0 + e], 0) * scale[(i0 + e) / K]);
+    }
+  }
 }
 
 __global__ void cast_e4m3fn_kernel(const float* __restrict__ in, int64_t n, uint8_t* __restrict__ out) {
@@ -424,7 +464,7 @@ hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t
     dequantize_rows_vec8_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const uint8_t*>(xq), scale, chunks, (int)(K / 8),
                                                       reinterpret_cast<uint16_t*>(out));
   } else {
-    const int64_t want = (total + 255) / 256;
+    const int64_t want = ((total + 7) / 8 + 255) / 256;
     const unsigned blocks = (unsigned)(want > 65536 ? 65536 : want);
     dequantize_rows_generic_kernel<<<blocks, 256, 0, s>>>(reinterpret_cast<const uint8_t*>(xq), scale, total, K,
                                                          reinterpret_cast<uint16_t*>(out));

@@ -216,7 +216,7 @@ def test_jagged_rows(shape, align, idx_dtype):
 
 
 @pytest.mark.parametrize("shape", [(1, 256), (3, 16), (7, 777), (64, 1024), (2, 3, 17, 136), (2500, 4096), (5, 3), (300, 4104),
-                                   (4096, 520), (33, 8), (1000, 1000)])
+                                   (4096, 520), (33, 8), (1000, 1000), (300, 4100), (33, 7), (2, 9), (513, 1001)])
 def test_dequantize_bit_exact(shape):
     g = torch.Generator().manual_seed(sum(shape))
     rows = 1
