@@ -134,8 +134,9 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
  * mslk_amd_f8f8bf16_rowwise_workspace_bytes(M,N,K) > 0, i.e. when K is not a multiple of 16: the call then copies both
  * operands into workspace rows of K rounded up to 16 (zero tail) and runs the MFMA kernels on the copies (the CK
  * instances of the reference pad K inside the kernel, fp8_rowwise_common.h:109-110 `GemmSpecialization::MNKPadding`).
- * Without a workspace (null or too small) such a K still gives the same results through a scalar kernel that is
- * orders of magnitude slower.  The workspace needs no initialisation and holds nothing between calls; calls that
+ * An operand base pointer that is not 16-byte aligned is handled the same way if the workspace holds
+ * (M + N) * round_up(K, 16) bytes.  Without a workspace (null or too small) such operands still give the same results
+ * through a scalar kernel that is orders of magnitude slower.  The workspace needs no initialisation and holds nothing between calls; calls that
  * share one workspace must not overlap.
  */
 int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,

@@ -168,10 +168,12 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
     return fail("%s: pre-shuffled weights need N %% 16 == 0 and K %% 64 == 0 (got N=%lld, K=%lld)", op, (long long)N, (long long)K);
   GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, bias, (uint16_t*)y,
                 (int)M, (int)N, (int)K, bias_dtype, out_f16, preshuffled};
-  const size_t pad_bytes = mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K);
-  if (pad_bytes > 0 && !preshuffled && workspace && workspace_bytes >= pad_bytes &&
+  // Operand rows the 16-byte loads cannot fetch (K % 16 != 0, or a base pointer that is not 16-byte aligned) are copied
+  // into the workspace when the caller gave one that holds both copies.
+  const int64_t Kp = (K + 15) / 16 * 16;
+  const bool unfetchable = K % 16 != 0 || reinterpret_cast<uintptr_t>(xq) % 16 != 0 || reinterpret_cast<uintptr_t>(wq) % 16 != 0;
+  if (unfetchable && !preshuffled && workspace && workspace_bytes >= (size_t)((M + N) * Kp) &&
       reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
-    const int64_t Kp = (K + 15) / 16 * 16;
     if (Kp <= kIntMax) {
       uint8_t* xp = static_cast<uint8_t*>(workspace);
       uint8_t* wp = xp + M * Kp;

@@ -129,7 +129,7 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, o
                 1 if out_dtype == torch.float16 else 0, M, N, K, _stream_ptr(XQ.device)))
         return Y
     wsp_ptr, wsp_bytes = None, 0
-    if K % 16:
+    if K % 16 or XQ.data_ptr() % 16 or WQ.data_ptr() % 16:
         # rows the 16-byte loads cannot fetch: room for copies with K rounded up (the caching allocator's block, so the
         # call stays capturable); the library pads into it and runs the MFMA kernels on the copies
         wsp_bytes = (M + N) * ((K + 15) // 16 * 16)

@@ -130,14 +130,27 @@ def test_out_variant_leading_dims_and_empty():
         torch.ops.mslk.f8f8bf16_rowwise(*_gpu(xq, wq, xs.half(), ws))
 
 
-def test_unaligned_views_take_the_generic_path():
+def test_unaligned_views_are_copied_or_take_the_generic_path():
+    from mslk_amd import _lib
     g = torch.Generator().manual_seed(23)
-    xq, wq, xs, ws = _random_problem(40, 72, 96, g)
-    buf = torch.empty(40 * 96 + 1, dtype=torch.uint8, device=DEV)
-    buf[1:] = xq.view(torch.uint8).reshape(-1).to(DEV)
-    xq_off = buf[1:].view(F8).view(40, 96)   # contiguous but only 1-byte aligned
-    y = torch.ops.mslk.f8f8bf16_rowwise(xq_off, *_gpu(wq, xs, ws))
-    assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws))
+    for (M, N, K) in [(40, 72, 96), (300, 1030, 1024)]:
+        xq, wq, xs, ws = _random_problem(M, N, K, g)
+        buf = torch.empty(M * K + 1, dtype=torch.uint8, device=DEV)
+        buf[1:] = xq.view(torch.uint8).reshape(-1).to(DEV)
+        xq_off = buf[1:].view(F8).view(M, K)   # contiguous but only 1-byte aligned
+        wbuf = torch.empty(N * K + 3, dtype=torch.uint8, device=DEV)
+        wbuf[3:] = wq.view(torch.uint8).reshape(-1).to(DEV)
+        wq_off = wbuf[3:].view(F8).view(N, K)
+        ref = O.dequant_matmul(xq, wq, xs, ws)
+        xs_d, ws_d = _gpu(xs, ws)
+        assert_gemm_close(torch.ops.mslk.f8f8bf16_rowwise(xq_off, wq.to(DEV), xs_d, ws_d), ref)      # via the workspace copy
+        assert_gemm_close(torch.ops.mslk.f8f8bf16_rowwise(xq.to(DEV), wq_off, xs_d, ws_d), ref)
+        assert_gemm_close(torch.ops.mslk.f8f8f16_rowwise(xq_off, wq_off, xs_d, ws_d), ref)
+        y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)                                        # no workspace: scalar kernel
+        _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise(xq_off.data_ptr(), wq_off.data_ptr(), xs_d.data_ptr(), ws_d.data_ptr(),
+                                                        None, 0, y.data_ptr(), M, N, K, None, 0, None))
+        torch.cuda.synchronize()
+        assert_gemm_close(y, ref)
 
 
 @pytest.mark.parametrize("M,N,K", [(300, 520, 1000), (1, 8192, 8200), (16, 8192, 8190), (64, 600, 17), (5, 7, 1), (512, 4096, 1001),
