@@ -150,20 +150,23 @@ MSLK_AMD_DEVINL uint2 quantize8_saturating(const float (&y)[8], float s) {
 
 // Vector path: D % 8 == 0, input rows 16-byte aligned, output rows 8-byte aligned.  NV > 0: the lane
 // keeps NV x 8 produced values in registers; NV == 0: rows of any length, produced twice.
-template <int OP, int DTYPE, int NV>
+// TEAM = 256: one workgroup per row; TEAM = 64: one wavefront per row, four rows per workgroup (rows of MoE
+// intermediate sizes, 768 ... 2048 elements, leave most of a 256-lane team idle).
+template <int OP, int DTYPE, int NV, int TEAM = 256>
 __global__ __launch_bounds__(256) void fused_quant_vec_kernel(FusedQuantArgs p) {
   __shared__ uint32_t smem[4];
-  const int64_t row = blockIdx.x;
-  const RowSource r = resolve_row<OP>(p, row);   // uniform over the workgroup
+  const int64_t row = TEAM == 256 ? (int64_t)blockIdx.x : (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (TEAM != 256 && row >= p.rows) return;      // uniform over the wavefront; this variant has no workgroup barrier
+  const RowSource r = resolve_row<OP>(p, row);   // uniform over the team
   if (!r.live) return;
   const int nvec = p.D >> 3;
-  const int lane = threadIdx.x;
+  const int lane = TEAM == 256 ? (int)threadIdx.x : (int)(threadIdx.x & 63);
   uint32_t m = 0;
   float cache[NV > 0 ? NV : 1][8];
   if constexpr (NV > 0) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int vec = i * 256 + lane;
+      const int vec = i * TEAM + lane;
       if (vec < nvec) {
         produce8<OP, DTYPE>(r, vec, cache[i]);
 #pragma unroll
@@ -171,14 +174,19 @@ __global__ __launch_bounds__(256) void fused_quant_vec_kernel(FusedQuantArgs p) 
       }
     }
   } else {
-    for (int vec = lane; vec < nvec; vec += 256) {
+    for (int vec = lane; vec < nvec; vec += TEAM) {
       float y[8];
       produce8<OP, DTYPE>(r, vec, y);
 #pragma unroll
       for (int e = 0; e < 8; ++e) m = max(m, __float_as_uint(y[e]) & 0x7FFFFFFFu);
     }
   }
-  m = block_max_bits(m, smem);
+  if constexpr (TEAM == 256) {
+    m = block_max_bits(m, smem);
+  } else {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, 64));
+  }
   float s, inv;
   row_scales(m, p.scale_ub, s, inv);
   if (lane == 0) p.out_scale[row] = inv;
@@ -186,14 +194,14 @@ __global__ __launch_bounds__(256) void fused_quant_vec_kernel(FusedQuantArgs p) 
   if constexpr (NV > 0) {
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
-      const int vec = i * 256 + lane;
+      const int vec = i * TEAM + lane;
       if (vec < nvec) {
         const uint2 q = quantize8_saturating(cache[i], s);
         __builtin_nontemporal_store(v2i{(int)q.x, (int)q.y}, reinterpret_cast<v2i*>(out_row + vec));
       }
     }
   } else {
-    for (int vec = lane; vec < nvec; vec += 256) {
+    for (int vec = lane; vec < nvec; vec += TEAM) {
       float y[8];
       produce8<OP, DTYPE>(r, vec, y);
       const uint2 q = quantize8_saturating(y, s);
@@ -229,6 +237,12 @@ hipError_t launch_fused_t(const FusedQuantArgs& p, hipStream_t s) {
                       reinterpret_cast<uintptr_t>(p.out) % 8 == 0;
   if (!vec_ok) {
     fused_quant_generic_kernel<OP, DTYPE><<<rows, 256, 0, s>>>(p);
+  } else if (p.D <= 2048 && p.rows >= 2048) {
+    // enough rows to fill the chip with one wavefront each
+    const unsigned blocks = (unsigned)((p.rows + 3) / 4);
+    if (p.D <= 512) fused_quant_vec_kernel<OP, DTYPE, 1, 64><<<blocks, 256, 0, s>>>(p);
+    else if (p.D <= 1024) fused_quant_vec_kernel<OP, DTYPE, 2, 64><<<blocks, 256, 0, s>>>(p);
+    else fused_quant_vec_kernel<OP, DTYPE, 4, 64><<<blocks, 256, 0, s>>>(p);
   } else if (p.D <= 2048) {
     fused_quant_vec_kernel<OP, DTYPE, 1><<<rows, 256, 0, s>>>(p);
   } else if (p.D <= 4096) {

@@ -33,6 +33,10 @@ def _code_distance(a, b):
     (300, 2048, None, True, False, torch.float16), (64, 16384, None, True, False, torch.bfloat16),
     (9, 20000, 1200.0, True, False, torch.bfloat16), (33, 1001, None, True, True, torch.bfloat16),
     (16384, 5120, None, False, False, torch.bfloat16),
+    # rows of MoE intermediate sizes in large numbers: one wavefront per row
+    (4099, 768, None, True, True, torch.bfloat16), (2048, 1408, 1200.0, False, False, torch.bfloat16),
+    (3001, 2048, None, True, False, torch.float16), (5000, 128, None, False, True, torch.bfloat16),
+    (2050, 520, 0.05, True, False, torch.bfloat16), (2047, 768, None, True, False, torch.bfloat16),
 ])
 def test_silu_mul_quant(T, D, ub, contiguous, partial, dtype):
     g = torch.Generator().manual_seed(T + D)
@@ -90,6 +94,10 @@ def test_silu_mul_quant_skips_invalid_rows_and_matches_two_step_path():
     (4, 300, 7168, False, True, torch.float16, torch.float16, torch.int64),
     (3, 40, 1001, False, True, torch.bfloat16, torch.float32, torch.int32),
     (2, 16, 20000, False, False, torch.bfloat16, torch.bfloat16, torch.int32),
+    (8, 4099, 768, True, False, torch.bfloat16, torch.bfloat16, torch.int32),
+    (4, 2048, 1408, False, True, torch.bfloat16, torch.float32, torch.int64),
+    (2, 3001, 2048, True, True, torch.float16, torch.float16, torch.int32),
+    (3, 6000, 136, False, False, torch.bfloat16, torch.bfloat16, torch.int32),
 ])
 def test_gather_scale_quant_bit_exact(E, T, D, partial, rowmajor, xdtype, sdtype, idx):
     g = torch.Generator().manual_seed(E * 1000 + T + D)
