@@ -146,6 +146,22 @@ int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_sca
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * mslk_amd_f8f8bf16_rowwise for callers that cannot allocate a workspace (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid allocation).  No counterpart in the reference.  Same arguments and results as
+ * mslk_amd_f8f8bf16_rowwise, but the padded operand copies of the K % 16 != 0 / unaligned-operand case go into a
+ * fixed array of MSLK_AMD_STATIC_SCRATCH_BYTES that is part of the library's device code (every GPU the library runs on
+ * holds it until the process ends); the call allocates and frees nothing.  Shapes whose copies do not fit,
+ * (M + N) * round_up(K, 16) > MSLK_AMD_STATIC_SCRATCH_BYTES, are rejected with an error.  The array needs no
+ * initialisation (the copies overwrite every byte they later read), but all calls on one GPU share it: calls that
+ * overlap on one GPU (different streams, or threads) race.  Shapes that need no copies never touch the array.
+ */
+#define MSLK_AMD_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
+int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                                             const void* bias, int bias_dtype, void* y,
+                                             int64_t M, int64_t N, int64_t K, void* stream);
+size_t mslk_amd_static_scratch_bytes(void);
+
+/*
  * The same GEMM with an fp16 (IEEE half, round to nearest even, overflow to infinity) output.
  * Replaces mslk::gemm::f8f8f16_rowwise (reference: csrc/gemm/gemm_ops.cpp:88-89,
  * csrc/gemm/ck/fp8_rowwise/fp8fp8fp16_rowwise_gemm.hip:66-133).  Arguments as above (the same workspace rule); y is fp16.

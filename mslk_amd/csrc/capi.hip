@@ -4,6 +4,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "../../include/mslk_amd.h"
 #include "kernels.h"
@@ -26,6 +27,32 @@ int check_hip(hipError_t e, const char* what) {
 }
 
 constexpr int64_t kIntMax = 2147483647;
+
+// Device memory for the padded operand copies of mslk_amd_f8f8bf16_rowwise_static_scratch: part of the code object, so
+// every GPU the library runs on holds its own copy from module load until the process ends.  In host code the name
+// below is only a handle for hipGetSymbolAddress; kernels and copies get the per-device address it returns.
+constexpr size_t kScratchBytes = MSLK_AMD_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device; looked up once per device, with that device current.
+int scratch_of_current_device(void** out) {
+  int dev = 0;
+  if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+  if (dev < 0 || dev >= kMaxDevices) return fail("static scratch: device index %d out of range", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    if (int rc = check_hip(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+    if (ptr == nullptr) return fail("static scratch: hipGetSymbolAddress returned a null address");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
 
 }  // namespace
 
@@ -198,6 +225,27 @@ int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_sca
                               const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
                               void* workspace, size_t workspace_bytes, void* stream) {
   return rowwise_impl("f8f8bf16_rowwise", 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, workspace, workspace_bytes, stream);
+}
+
+size_t mslk_amd_static_scratch_bytes(void) { return kScratchBytes; }
+
+int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
+                                             const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                                             void* stream) {
+  const char* op = "f8f8bf16_rowwise_static_scratch";
+  void* ptr = nullptr;
+  size_t bytes = 0;
+  const bool unfetchable = K % 16 != 0 || reinterpret_cast<uintptr_t>(xq) % 16 != 0 || reinterpret_cast<uintptr_t>(wq) % 16 != 0;
+  if (M > 0 && N > 0 && K > 0 && M <= kIntMax && N <= kIntMax && K <= kIntMax && unfetchable) {
+    const int64_t Kp = (K + 15) / 16 * 16;
+    const double need = ((double)M + (double)N) * (double)Kp;
+    if (need > (double)kScratchBytes)
+      return fail("%s: the padded operand copies need (M + N) * round_up(K, 16) = %.0f bytes, the static scratch array holds %zu; "
+                  "use mslk_amd_f8f8bf16_rowwise with a workspace", op, need, kScratchBytes);
+    if (int rc = scratch_of_current_device(&ptr)) return rc;
+    bytes = kScratchBytes;
+  }
+  return rowwise_impl(op, 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, ptr, bytes, stream);
 }
 
 int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,

@@ -1,0 +1,80 @@
+"""The entry point that allocates nothing: mslk_amd_f8f8bf16_rowwise_static_scratch.
+
+It must give the bits of mslk_amd_f8f8bf16_rowwise called with a caller-allocated workspace, on two calls in a row that
+share the library's static scratch array (the second smaller, so stale bytes of the first call lie behind its copies),
+and reject shapes whose padded copies do not fit.  Collected last, so that a failure here hides no other test.
+"""
+import pytest
+import torch
+
+from mslk_amd import _lib
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _operands(M, N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    xq = torch.randint(0, 256, (M, K), generator=g, dtype=torch.uint8)
+    wq = torch.randint(0, 256, (N, K), generator=g, dtype=torch.uint8)
+    # no NaN codes (0x7F / 0xFF): the comparison below is bitwise on finite outputs
+    xq[(xq & 0x7F) == 0x7F] = 0x30
+    wq[(wq & 0x7F) == 0x7F] = 0x30
+    xs = torch.rand(M, generator=g) * 0.01 + 1e-3
+    ws = torch.rand(N, generator=g) * 0.01 + 1e-3
+    bias = (torch.randn(N, generator=g) * 0.1).bfloat16()
+    return [t.to(DEV) for t in (xq, wq, xs, ws, bias)]
+
+
+def _with_workspace(xq, wq, xs, ws, bias, M, N, K):
+    L = _lib.lib()
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    nbytes = L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+    wsp = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(L.mslk_amd_f8f8bf16_rowwise(xq.data_ptr(), wq.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias.data_ptr(), 2,
+                                           y.data_ptr(), M, N, K, wsp.data_ptr(), nbytes, stream))
+    return y
+
+
+def _static(xq, wq, xs, ws, bias, M, N, K):
+    L = _lib.lib()
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    stream = torch.cuda.current_stream().cuda_stream
+    _lib.check(L.mslk_amd_f8f8bf16_rowwise_static_scratch(xq.data_ptr(), wq.data_ptr(), xs.data_ptr(), ws.data_ptr(),
+                                                          bias.data_ptr(), 2, y.data_ptr(), M, N, K, stream))
+    return y
+
+
+def test_static_scratch_matches_the_workspace_entry_point_on_two_calls():
+    # K % 16 != 0: both operands are copied into padded rows.  First a larger problem, then a smaller one whose copies
+    # occupy the front of the bytes the first call left behind.
+    for i, (M, N, K) in enumerate([(300, 1000, 1001), (17, 264, 200)]):
+        print(f"static scratch case {i}: M={M} N={N} K={K}", flush=True)
+        ops = _operands(M, N, K, seed=50 + i)
+        want = _with_workspace(*ops, M, N, K)
+        got = _static(*ops, M, N, K)
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16).cpu(), want.view(torch.int16).cpu()), f"case {i}: outputs differ"
+
+
+def test_static_scratch_aligned_shapes_do_not_need_the_array():
+    M, N, K = 64, 512, 1024
+    ops = _operands(M, N, K, seed=7)
+    want = _with_workspace(*ops, M, N, K)
+    got = _static(*ops, M, N, K)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16).cpu(), want.view(torch.int16).cpu())
+
+
+def test_static_scratch_rejects_what_does_not_fit():
+    L = _lib.lib()
+    cap = L.mslk_amd_static_scratch_bytes()
+    assert cap == 32 << 20
+    M, N, K = 4096, 4096, 4100          # (M + N) * 4112 bytes > 32 MiB
+    assert (M + N) * ((K + 15) // 16 * 16) > cap
+    # never dereferenced: the size check comes first
+    rc = L.mslk_amd_f8f8bf16_rowwise_static_scratch(16, 16, 16, 16, None, 0, 16, M, N, K, None)
+    assert rc != 0
+    msg = L.mslk_amd_last_error().decode()
+    assert "static scratch" in msg and "workspace" in msg
