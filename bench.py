@@ -168,9 +168,9 @@ def _vendor_sweep(api):
     for (N, K) in [(8192, 8192), (10240, 8192), (57344, 8192), (8192, 28672), (4096, 4096), (6144, 4096), (28672, 4096), (4096, 14336)]:
         nsets = 6 if N * K < 2 ** 27 else 3
         g = torch.Generator(device=dev).manual_seed(N + K)
-        weights = [mslk_amd.quantize_fp8_row(torch.randn(N, K, device=dev, generator=g).bfloat16()) for _ in range(nsets)]
+        weights = [mslk_amd.quantize_fp8_row(torch.randn(N, K, device=dev, generator=g).bfloat16(), use_triton=False) for _ in range(nsets)]
         for M in (1, 16, 64, 128, 256, 384, 512, 1024, 2048, 4096, 8192, 16384):
-            acts = [mslk_amd.quantize_fp8_row(torch.randn(M, K, device=dev, generator=g).bfloat16()) for _ in range(nsets)]
+            acts = [mslk_amd.quantize_fp8_row(torch.randn(M, K, device=dev, generator=g).bfloat16(), use_triton=False) for _ in range(nsets)]
             ys = [torch.empty(M, N, dtype=torch.bfloat16, device=dev) for _ in range(nsets)]
 
             def ours(i):
@@ -232,8 +232,8 @@ def main():
     M, K = wl.x.shape
     N = wl.w.shape[0]
     x_dev = wl.x.to(dev)
-    wq0, ws0 = mslk_amd.quantize_fp8_row(wl.w.to(dev))
-    xq0, xs0 = mslk_amd.quantize_fp8_row(x_dev)
+    wq0, ws0 = mslk_amd.quantize_fp8_row(wl.w.to(dev), use_triton=False)
+    xq0, xs0 = mslk_amd.quantize_fp8_row(x_dev, use_triton=False)
     NSETS = 6  # 6 x (16 + 16 + 32 MiB) = 384 MiB of distinct operands > 256 MB Infinity Cache
     sets = [(xq0.clone(), wq0.clone(), xs0.clone(), ws0.clone(), torch.empty(M, N, dtype=torch.bfloat16, device=dev))
             for _ in range(NSETS)]
@@ -378,13 +378,13 @@ def main():
     # ---------------------------------------------------------------- decode sweep (cfg3)
     if (not args.no_extras and args.only == "") or args.only == "decode":
         Nd = Kd = 8192
-        wq3, ws3 = mslk_amd.quantize_fp8_row(W.cfg3_weight().to(dev))
+        wq3, ws3 = mslk_amd.quantize_fp8_row(W.cfg3_weight().to(dev), use_triton=False)
         wsets = [wq3.clone() for _ in range(6)]  # 6 x 64 MiB > Infinity Cache
         wshuf = [mslk_amd.preshuffle_b_mfma(w) for w in wsets]   # the same weights in the pre-shuffled (blocked) layout
         decode = {}
         for Md in (1, 4, 16, 64):
             xd = W.cfg3_activations(Md).to(dev)
-            xq3, xs3 = mslk_amd.quantize_fp8_row(xd)
+            xq3, xs3 = mslk_amd.quantize_fp8_row(xd, use_triton=False)
             y3 = torch.empty(Md, Nd, dtype=torch.bfloat16, device=dev)
 
             def dec_step(i):
@@ -420,15 +420,15 @@ def main():
     # ---------------------------------------------------------------- other configs (GEMM rate only)
     if not args.no_extras:
         wl0 = W.cfg0()
-        a, sa = mslk_amd.quantize_fp8_row(wl0.x.to(dev))
-        b, sb = mslk_amd.quantize_fp8_row(wl0.w.to(dev))
+        a, sa = mslk_amd.quantize_fp8_row(wl0.x.to(dev), use_triton=False)
+        b, sb = mslk_amd.quantize_fp8_row(wl0.w.to(dev), use_triton=False)
         y0 = torch.empty(1024, 1024, dtype=torch.bfloat16, device=dev)
         ms = _median_events_ms(lambda i: api.gemm(a, b, sa, sb, y0), 100)
         extras["gemm_cfg0_1024"] = {"ms": ms, "TFLOPs": 2.0 * 1024**3 / (ms * 1e-3) / 1e12}
 
         wl2 = W.cfg2()
-        a, sa = mslk_amd.quantize_fp8_row(wl2.x.to(dev))
-        b, sb = mslk_amd.quantize_fp8_row(wl2.w.to(dev))
+        a, sa = mslk_amd.quantize_fp8_row(wl2.x.to(dev), use_triton=False)
+        b, sb = mslk_amd.quantize_fp8_row(wl2.w.to(dev), use_triton=False)
         bias2 = wl2.bias.to(dev)
         y2 = torch.empty(8192, 28672, dtype=torch.bfloat16, device=dev)
         for _ in range(30):
@@ -440,10 +440,10 @@ def main():
         del a, b, y2, wl2
 
         wl4 = W.cfg4()
-        xq4, xs4 = mslk_amd.quantize_fp8_row(wl4.x.to(dev))
+        xq4, xs4 = mslk_amd.quantize_fp8_row(wl4.x.to(dev), use_triton=False)
         wq4, ws4 = [], []
         for w in wl4.w:
-            q, s = mslk_amd.quantize_fp8_row(w.to(dev))
+            q, s = mslk_amd.quantize_fp8_row(w.to(dev), use_triton=False)
             wq4.append(q)
             ws4.append(s)
         xl, sl = list(xq4.split(wl4.counts)), list(xs4.split(wl4.counts))

@@ -12,7 +12,7 @@
  *   WQ  [N, K]  e4m3fn codes, row-major contiguous          (weights; i.e. B is column-major, "TN")
  *   x_scale [M], w_scale [N]  fp32
  *   bias [N]  fp32 or bf16, optional
- *   Y   [M, N]  bf16, row-major contiguous:  Y = bf16( acc_fp32 * x_scale[m] * w_scale[n] + bias[n] )
+ *   Y   [M, N]  bf16, row-major contiguous:  Y = bf16( (acc_fp32 * w_scale[n]) * x_scale[m] + bias[n] )
  */
 #ifndef MSLK_AMD_H_
 #define MSLK_AMD_H_
@@ -218,7 +218,7 @@ int mslk_amd_f8f8bf16_rowwise_grouped_stacked(const void* xq, const void* wq, co
 /*
  * Grouped GEMM in the torch._grouped_mm calling convention: group boundaries are int32 cumulative
  * END offsets in DEVICE memory (no host sync; graph-safe).  Replaces
- * mslk::gemm::f8f8bf16_rowwise_grouped_mm (reference: csrc/gemm/gemm_ops.cpp:35-36,
+ * mslk::gemm::f8f8bf16_rowwise_grouped_mm (reference: csrc/gemm/gemm_ops.cpp:95-96,
  * csrc/gemm/ck/fp8_rowwise_grouped/fp8_rowwise_grouped_gemm.hip:720-845; the per-group pointer
  * arithmetic restates set_kernel_args, same file 161-296).  `layout` selects the varying dimension;
  * M, N, K are the full tensor extents (the varying one is the total over groups):
@@ -256,7 +256,7 @@ int mslk_amd_f8f8bf16_rowwise_grouped_dynamic(const void* xq, const void* wq, co
 
 /*
  * Batched rowwise FP8 GEMM: Y[b] = bf16(XQ[b] . WQ[b]^T * x_scale[b][:,None] * w_scale[b][None,:] + bias[b]).
- * Replaces mslk::gemm::f8f8bf16_rowwise_batched (reference: csrc/gemm/gemm_ops.cpp:95-96,
+ * Replaces mslk::gemm::f8f8bf16_rowwise_batched (reference: csrc/gemm/gemm_ops.cpp:35-36,
  * csrc/gemm/ck/fp8_rowwise_batched/fp8_rowwise_batched_gemm.hip:199-254).
  *   xq [B, M, K], wq [B, N, K], x_scale [B, M], w_scale [B, N], bias NULL or [B, N] (layout of
  *   csrc/gemm/cutlass/f8f8bf16_rowwise_batched/f8f8bf16_rowwise_batched_common.cuh:272-275), y [B, M, N].

@@ -6,7 +6,7 @@ Importing the package registers `torch.ops.mslk.f8f8bf16_rowwise`, `..._rowwise_
 `torch.ops.mslk.quantize_fp8_row` / `dequantize_fp8_row`, all backed by hand-written HIP kernels in libmslk_amd.so.
 """
 from . import _lib  # noqa: F401
-from .quantize import (quantize_fp8_row, quantize_fp8_per_row, dequantize_fp8_row, set_quantize_numerics,  # noqa: F401
+from .quantize import (quantize_fp8_row, quantize_fp8_per_row, dequantize_fp8_row,  # noqa: F401
                        FP8_DTYPE)  # noqa: F401
 from . import gemm  # noqa: F401  (registers torch.ops.mslk.*)
 from . import moe  # noqa: F401  (registers torch.ops.mslk.silu_mul_quant / gather_scale_quant_dense_tokens)
@@ -17,6 +17,6 @@ from .gemm import (f8f8bf16_rowwise, f8f8bf16_rowwise_out, f8f8f16_rowwise, f8f8
                    f8f8bf16_rowwise_grouped_mm, f8f8bf16_rowwise_grouped_dynamic,
                    f8f8bf16_rowwise_batched)
 
-__all__ = ["quantize_fp8_row", "quantize_fp8_per_row", "dequantize_fp8_row", "set_quantize_numerics", "silu_mul_quant", "gather_scale_quant_dense_tokens", "f8f8bf16_rowwise", "f8f8bf16_rowwise_out", "f8f8f16_rowwise", "f8f8bf16_rowwise_preshuffle", "f8f8f16_rowwise_preshuffle", "preshuffle_b_mfma", "ck_preshuffle",
+__all__ = ["quantize_fp8_row", "quantize_fp8_per_row", "dequantize_fp8_row", "silu_mul_quant", "gather_scale_quant_dense_tokens", "f8f8bf16_rowwise", "f8f8bf16_rowwise_out", "f8f8f16_rowwise", "f8f8bf16_rowwise_preshuffle", "f8f8f16_rowwise_preshuffle", "preshuffle_b_mfma", "ck_preshuffle",
            "f8f8bf16_rowwise_grouped", "f8f8bf16_rowwise_grouped_cat", "f8f8bf16_rowwise_grouped_stacked",
            "f8f8bf16_rowwise_grouped_mm", "f8f8bf16_rowwise_grouped_dynamic", "f8f8bf16_rowwise_batched", "FP8_DTYPE"]

@@ -160,7 +160,7 @@ __global__ __launch_bounds__(256) void generic_kernel(GemmProblem p) {
     for (int k = 0; k < p.K; ++k)
       acc += __builtin_amdgcn_cvt_f32_fp8((int)a[k], 0) * __builtin_amdgcn_cvt_f32_fp8((int)b[k], 0);
   }
-  float v = (acc * p.xs[m]) * p.ws[n];
+  float v = (acc * p.ws[n]) * p.xs[m];
   if (p.bias_dtype == 1) v += reinterpret_cast<const float*>(p.bias)[n];
   else if (p.bias_dtype == 2) v += bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[n]);
   p.y[idx] = (uint16_t)f32_to_out_bits(v, p.out_f16);

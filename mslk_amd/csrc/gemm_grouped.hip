@@ -167,7 +167,7 @@ MSLK_AMD_DEVINL void slow_tile(const uint8_t* a, const uint8_t* b, const float* 
     float acc = 0.f;
     for (int k = 0; k < K; ++k)
       acc += __builtin_amdgcn_cvt_f32_fp8((int)ar[k], 0) * __builtin_amdgcn_cvt_f32_fp8((int)br[k], 0);
-    float v = (acc * xs[m]) * ws[n];
+    float v = (acc * ws[n]) * xs[m];
     if constexpr (BIAS == 1) v += static_cast<const float*>(bias)[n];
     if constexpr (BIAS == 2) v += bf16_bits_to_f32(static_cast<const uint16_t*>(bias)[n]);
     y[(int64_t)m * ldc + n] = (uint16_t)f32_to_bf16_bits(v);

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) sum += red[w][tn][tm][t];
-    float val = (sum * e_xs[r]) * e_ws[r];
+    float val = (sum * e_ws[r]) * e_xs[r];
     if constexpr (BIAS != 0) val += e_b[r];
     p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_out_bits(val, p.out_f16);
   }
@@ -357,7 +357,7 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
     float sum = 0.f;
 #pragma unroll
     for (int w = 0; w < kWaves; ++w) sum += reinterpret_cast<const float*>(lds + w * XBUF)[frag * 256 + t];
-    float val = (sum * e_xs[r]) * e_ws[r];
+    float val = (sum * e_ws[r]) * e_xs[r];
     if constexpr (BIAS != 0) val += e_b[r];
     p.y[(int64_t)m * p.N + n] = (uint16_t)f32_to_out_bits(val, p.out_f16);
   }
@@ -378,7 +378,8 @@ hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
 
 bool skinny_supports(const GemmProblem& p) {
   if (p.w_preshuffled && (p.N % 16 != 0 || p.K % 64 != 0)) return false;
-  return p.M >= 1 && p.M <= 64 && p.K % 16 == 0 && p.K >= 16 &&
+  // the kernels form 32-bit byte offsets of up to 64 rows x K
+  return p.M >= 1 && p.M <= 64 && p.K % 16 == 0 && p.K >= 16 && (int64_t)64 * p.K < (int64_t(1) << 32) &&
          reinterpret_cast<uintptr_t>(p.xq) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0;
 }
 

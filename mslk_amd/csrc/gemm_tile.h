@@ -17,6 +17,11 @@
 //     load fetches logical chunk (l & 7) ^ swz(row) of its row.
 //   * Two XQ buffers and three WQ buffers: while step k is multiplied, the XQ tile of step k+1 and the
 //     WQ tiles of steps k+1 and k+2 are in flight (the weights are the cold, read-once stream).
+// Rows
+//   * The 16-row m fragments of a tile are dealt to the wave rows round-robin (wave row wm owns fragments wm, wm + WM,
+//     ...), and a tile with fewer valid rows than BM skips the MFMAs, the fragment reads, the DMA loads and the epilogue
+//     work of fragments that hold no valid row: the cost of a ragged tile (the last row tile of an MoE group) follows its
+//     row count in steps of 16 * WM rows, down to what the weight stream alone costs.
 // Math
 //   * v_mfma_f32_16x16x128_f8f6f4 (both operands e4m3, unit block scales).  WQ rows are the first
 //     operand and XQ rows the second, so a lane ends up holding 4 consecutive n for one m.
@@ -89,6 +94,8 @@ struct GemmTile {
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
   uint32_t b_off[TS::LB];
   int out_f16 = 0;          // output element type: 0 bf16, 1 fp16 (set by the caller before run())
+  int a_rows = TS::kBM;     // valid rows of the XQ tile (wave-uniform); DMA loads of 8-row groups beyond them are skipped
+  int fmv = TS::FM;         // m fragments of this wave that hold at least one valid row (wave-uniform)
   const uint8_t* a_base;    // XQ + m0 * K   (wave-uniform)
   const uint8_t* b_base;    // WQ + n0 * K
 
@@ -100,6 +107,12 @@ struct GemmTile {
     const int wave = wave_id();
     a_base = xq_tile;
     b_base = wq_tile;
+    a_rows = rows_a;
+    {
+      const int nf = (rows_a + 15) >> 4;                      // fragments of the tile with a valid row
+      const int mine = (nf - wave / TS::WN + TS::WM - 1) / TS::WM;   // of which this wave row owns fragments wm, wm + WM, ...
+      fmv = mine < 0 ? 0 : (mine > TS::FM ? TS::FM : mine);
+    }
 #pragma unroll
     for (int i = 0; i < TS::LA; ++i) {
       const int row = (wave * TS::LA + i) * 8 + (lane >> 3);
@@ -129,16 +142,20 @@ struct GemmTile {
 
   // DMA load number i (0 .. LA-1 for the XQ tile, 0 .. LB-1 for the WQ tile) of the K step at byte k0.
   // `abuf` / `bbuf` are the LDS buffers that receive the XQ / WQ tile of the K step at byte k0.
+  // RAGGED: the 8 rows of a load that lie beyond the valid rows of the tile are not fetched (nobody multiplies them).
+  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void issue_a(char* abuf, int k0, int i) {
+    if (RAGGED && (wave_id() * TS::LA + i) * 8 >= a_rows) return;   // wave-uniform
     dma16(a_base + k0 + a_off[i], abuf + (wave_id() * TS::LA + i) * 1024);
   }
   MSLK_AMD_DEVINL void issue_b(char* bbuf, int k0, int i) {
     // pre-shuffled: the K step at byte k0 starts 16 rows x k0 bytes into the row group
     dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
   }
+  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void issue_a_all(char* abuf, int k0) {
 #pragma unroll
-    for (int i = 0; i < TS::LA; ++i) issue_a(abuf, k0, i);
+    for (int i = 0; i < TS::LA; ++i) issue_a<RAGGED>(abuf, k0, i);
   }
   MSLK_AMD_DEVINL void issue_b_all(char* bbuf, int k0) {
 #pragma unroll
@@ -179,11 +196,15 @@ struct GemmTile {
     const int c0 = PS ? g : 2 * g, c1 = PS ? g + 4 : 2 * g + 1;
     return FragOff{i * kBK + ((c0 ^ s) << 4), i * kBK + ((c1 ^ s) << 4)};
   }
+  // Fragment t of a wave: STRIDE bytes after fragment t - 1 (consecutive 16-row blocks for WQ; every WM-th for XQ).
+  template <int STRIDE = 16 * kBK>
   MSLK_AMD_DEVINL static v8i load_frag(const char* tile, int t, FragOff fo) {
-    const v4i lo = *reinterpret_cast<const v4i*>(tile + t * 16 * kBK + fo.off0);
-    const v4i hi = *reinterpret_cast<const v4i*>(tile + t * 16 * kBK + fo.off1);
+    const v4i lo = *reinterpret_cast<const v4i*>(tile + t * STRIDE + fo.off0);
+    const v4i hi = *reinterpret_cast<const v4i*>(tile + t * STRIDE + fo.off1);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
+  static constexpr int A_FRAG_STRIDE = TS::WM * 16 * kBK;   // wave row wm owns the m fragments wm, wm + WM, ...
+  MSLK_AMD_DEVINL static v8i load_frag_a(const char* tile, int t, FragOff fo) { return load_frag<A_FRAG_STRIDE>(tile, t, fo); }
   // WQ fragment t of the wave: as load_frag, or lane-linear out of the two 1 KiB blocks of row group t.
   MSLK_AMD_DEVINL static v8i load_frag_b(const char* tile, int t, FragOff fo) {
     if constexpr (PS) {
@@ -197,17 +218,19 @@ struct GemmTile {
   }
   // The part of an XQ / WQ buffer this wave multiplies.
   MSLK_AMD_DEVINL static const char* a_tile_of(const char* abuf) {
-    return abuf + (wave_id() / TS::WN) * (TS::kBM / TS::WM) * kBK;
+    return abuf + (wave_id() / TS::WN) * 16 * kBK;
   }
   MSLK_AMD_DEVINL static const char* b_tile_of(const char* bbuf) {
     return bbuf + (wave_id() % TS::WN) * (TS::kBN / TS::WN) * kBK;
   }
   // First fragments of a K step: all XQ fragments and WQ fragment 0.
+  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void load_first_frags(const char* abuf, const char* bbuf, v8i (&xf)[TS::FM], v8i& wf0) {
     const FragOff fo = frag_off();
     wf0 = load_frag_b(b_tile_of(bbuf), 0, fo);
 #pragma unroll
-    for (int tm = 0; tm < TS::FM; ++tm) xf[tm] = load_frag(a_tile_of(abuf), tm, fo);
+    for (int tm = 0; tm < TS::FM; ++tm)
+      if (!RAGGED || tm < fmv) xf[tm] = load_frag_a(a_tile_of(abuf), tm, fo);
   }
 
   // Waits until at most `pending` of this wave's DMA loads (the youngest ones) are still in flight and
@@ -240,7 +263,9 @@ struct GemmTile {
   //     fragments already on their way.
   // In the symmetric ring (TileShape::RING) the XQ loads go to `a_dst` != `a_nxt` as well, and PENDING, the
   // number of this wave's youngest loads that may still be in flight at the barrier, covers RING - 2 steps.
-  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING>
+  // RAGGED: the tile has fewer than BM valid rows; MFMAs and XQ fragment reads of this wave's fragments >= fmv are
+  // skipped (wave-uniform branches) and so are the DMA loads of XQ rows nobody multiplies.
+  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING, bool RAGGED = false>
   MSLK_AMD_DEVINL void step(const char* b_cur, char* a_dst, const char* a_nxt, const char* b_nxt, char* b_far, int k_a,
                             int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
     constexpr int HALF = TS::FN / 2;
@@ -261,7 +286,8 @@ struct GemmTile {
       v8i wf_next;
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) {
-        acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+        if (!RAGGED || tm < fmv)
+          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
         if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
         const int d = tm - (TS::FM - SLOTS);
         if (tn < HALF && d >= 0) {
@@ -270,7 +296,7 @@ struct GemmTile {
             const int q = tn * NDMA + d * PER_SLOT + j;   // all XQ loads are older than all WQ loads of the step
             if (d * PER_SLOT + j < NDMA) {
               if (q < TS::LA) {
-                if constexpr (DMA_A) issue_a(a_dst, k_a, q);
+                if constexpr (DMA_A) issue_a<RAGGED>(a_dst, k_a, q);
               } else {
                 if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
               }
@@ -289,11 +315,11 @@ struct GemmTile {
     const char* a_next = a_tile_of(a_nxt);
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
-      acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
-      if constexpr (NEXT) {
-        xf[tm] = load_frag(a_next, tm, fo);
-        __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
+      if (!RAGGED || tm < fmv) {
+        acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+        if constexpr (NEXT) xf[tm] = load_frag_a(a_next, tm, fo);
       }
+      if constexpr (NEXT) __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -310,32 +336,40 @@ struct GemmTile {
                            const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K,
                            uint32_t ld) {
     v4f acc[TS::FN][TS::FM];
-    accumulate(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    // A tile with fewer valid rows than BM takes the K loop that skips the fragments without valid rows.
+    if constexpr (TS::RING == 0) {
+      if (m_rem < TS::kBM) accumulate<true>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+      else accumulate<false>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    } else {
+      accumulate<false>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    }
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
   }
 
   // K loop only: acc = sum over the K bytes of the operand rows starting at xq_tile / wq_tile.  Ends with a
   // workgroup barrier, after which the LDS buffers are dead.
+  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void accumulate(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
                                   uint32_t ld, v4f (&acc)[TS::FN][TS::FM]) {
     if constexpr (TS::RING == 0) {
-      prologue(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld);
+      prologue<RAGGED>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld);
     } else {
       init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
     }
-    accumulate_issued<false>(lds, K, acc);
+    accumulate_issued<false, RAGGED>(lds, K, acc);
   }
 
   // Two-plus-three buffers only: per-lane addresses of a tile and the first DMA loads of its K loop (step 0 of both
   // operands, step 1 of WQ) into the buffers the loop starts from.  A persistent workgroup calls this for its next
   // tile before the epilogue of the current one, which must then stay out of those three buffers.
+  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void prologue(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
                                 uint32_t ld) {
     static_assert(TS::RING == 0, "the symmetric ring issues its own prologue");
     init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
     const int KT = K / kBK;
     if (KT > 0) {
-      issue_a_all(lds, 0);
+      issue_a_all<RAGGED>(lds, 0);
       issue_b_all(lds + 2 * TS::A_BYTES, 0);
       if (KT > 1) issue_b_all(lds + 2 * TS::A_BYTES + TS::B_BYTES, kBK);
     }
@@ -344,8 +378,9 @@ struct GemmTile {
   // K loop after prologue() (or, for the symmetric ring, after init()).  DRAIN: the wave has other memory
   // operations in flight behind the prologue loads (the stores of the previous tile's epilogue), so the first wait
   // is for all of them instead of "all but the youngest WQ loads".
-  template <bool DRAIN>
+  template <bool DRAIN, bool RAGGED = false>
   MSLK_AMD_DEVINL void accumulate_issued(char* lds, int K, v4f (&acc)[TS::FN][TS::FM]) {
+    static_assert(!RAGGED || TS::RING == 0, "row skipping is built for the two-plus-three buffer tiles");
 #pragma unroll
     for (int tn = 0; tn < TS::FN; ++tn)
 #pragma unroll
@@ -365,19 +400,19 @@ struct GemmTile {
       if (KT > 0) {
         if (KT > 1 && !DRAIN) wait_and_barrier<TS::LB>();
         else wait_and_barrier<0>();
-        load_first_frags(a_cur, b_cur, xf, wf0);
+        load_first_frags<RAGGED>(a_cur, b_cur, xf, wf0);
         // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
         for (int kt = 0; kt < KT - 2; ++kt) {
-          step<true, true, true, TS::LB>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
+          step<true, true, true, TS::LB, RAGGED>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
         if (KT > 1) {
-          step<true, false, true, 0>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
+          step<true, false, true, 0, RAGGED>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
-        step<false, false, false, 0>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
+        step<false, false, false, 0, RAGGED>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
       }
     } else {
       // Symmetric ring: buffer i % RING holds step i; step kt fetches step kt + RING - 1 into the buffers step
@@ -419,8 +454,8 @@ struct GemmTile {
       __syncthreads();   // everybody is done with the buffers of the full steps before one pair is refilled
       issue_loads_tail(a_tail, b_tail, KT * kBK, k_tail);
       __syncthreads();
-      load_first_frags(a_tail, b_tail, xf, wf0);
-      step<false, false, false, 0>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
+      load_first_frags<RAGGED>(a_tail, b_tail, xf, wf0);
+      step<false, false, false, 0, RAGGED>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
     }
     __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
   }
@@ -480,7 +515,16 @@ struct GemmTile {
     constexpr int ROWS_W = TS::kBM / TS::WM;     // rows per wave
     static_assert(2 * BUF + ROWS_W * 4 == EPI_WAVE_BYTES, "epilogue buffer size");
     const int n_base = wn * WN;
-    const int m_base = wm * (TS::kBM / TS::WM);
+    // tile row of row j of this wave's m fragment tm (the fragments of a tile are dealt to the wave rows round-robin)
+    auto frag_row = [&](int tm) { return (tm * TS::WM + wm) * 16; };
+    // fragments of this wave with at least one valid row (formed from m_rem: a persistent workgroup has already run
+    // init() for its next tile when the epilogue of the current one starts)
+    int fm_live = TS::FM;
+    if constexpr (!ALL_ROWS) {
+      const int nf = ((m_rem < TS::kBM ? m_rem : TS::kBM) + 15) >> 4;
+      const int mine = (nf - wm + TS::WM - 1) / TS::WM;
+      fm_live = mine < 0 ? 0 : (mine > TS::FM ? TS::FM : mine);
+    }
     const bool vec_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
     const bool pair_store = (N & 1) == 0 && (reinterpret_cast<uintptr_t>(y) & 3) == 0;
 
@@ -530,7 +574,8 @@ struct GemmTile {
 #pragma unroll
     for (int i = 0; i < (ROWS_W + 63) / 64; ++i) {
       const int r = lane + i * 64;
-      if (ROWS_W % 64 == 0 || r < ROWS_W) xs_lds[r] = (ALL_ROWS || m_base + r < m_rem) ? xs[m_base + r] : 0.f;
+      const int row = frag_row(r >> 4) + (r & 15);
+      if (ROWS_W % 64 == 0 || r < ROWS_W) xs_lds[r] = (ALL_ROWS || row < m_rem) ? xs[row] : 0.f;
     }
 
     // Scale, convert and park n fragments [tn0, tn1) of fragment row tm in transpose buffer tm & 1.
@@ -547,7 +592,7 @@ struct GemmTile {
           float a;
           if constexpr (ACC_IN_AGPRS) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[tn][tm][r]));   // volatile: stays behind the s_nop
           else a = acc[tn][tm][r];
-          v[r] = (a * xsv) * wsv[tn][r];
+          v[r] = (a * wsv[tn][r]) * xsv;   // w_scale first, then x_scale: the order of the reference's epilogue (fp8_rowwise_common.h:66)
           if constexpr (BIAS != 0) v[r] += bv[tn][r];
         }
         uint2 pk;
@@ -566,7 +611,7 @@ struct GemmTile {
     };
     // Wave-uniform 64-bit row base + one 32-bit lane offset that is the same for every store of the tile.
     auto dst_of = [&](int tm, int pass) {
-      return reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(y + (int64_t)(m_base + tm * 16 + pass * RPI) * N) + lane_off);
+      return reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(y + (int64_t)(frag_row(tm) + pass * RPI) * N) + lane_off);
     };
 
     if constexpr (FULL) {
@@ -577,39 +622,46 @@ struct GemmTile {
       // vector ALU work side by side.
       static_assert(TS::FN % NP == 0, "whole n fragments per store");
       uint4 val[NP];
-      // consecutive store instructions of a wave are RPI rows apart: one 64-bit add per store
-      char* dst = reinterpret_cast<char*>(y + (int64_t)m_base * N) + lane_off;
+      // consecutive store instructions of a fragment are RPI rows apart, consecutive fragments of a wave 16 * WM rows:
+      // one 64-bit add per store
+      char* dst = reinterpret_cast<char*>(y + (int64_t)frag_row(0) * N) + lane_off;
       const int64_t dst_step = (int64_t)RPI * N * 2;
+      const int64_t frag_step = (int64_t)(TS::WM - 1) * 16 * N * 2;
       float xsv = xs_lds[j];
 #pragma unroll
       for (int tm = 0; tm <= TS::FM; ++tm) {
-        if (tm > 0) fetch(tm - 1, val);
+        // ragged tiles: fragments without a valid row are neither scaled nor stored (wave-uniform tests)
+        const bool do_park = tm < TS::FM && (ALL_ROWS || tm < fm_live);
+        const bool do_store = tm > 0 && (ALL_ROWS || tm - 1 < fm_live);
+        if (do_store) fetch(tm - 1, val);
         const float xsv_next = tm + 1 < TS::FM ? xs_lds[(tm + 1) * 16 + j] : 0.f;   // read one fragment row ahead
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int pass = 0; pass < NP; ++pass) {
-          if (tm < TS::FM) park(tm, pass * (TS::FN / NP), (pass + 1) * (TS::FN / NP), xsv);
+          if (do_park) park(tm, pass * (TS::FN / NP), (pass + 1) * (TS::FN / NP), xsv);
           __builtin_amdgcn_sched_barrier(0);
           if (tm > 0) {
-            const int r0 = m_base + (tm - 1) * 16 + pass * RPI;   // first of the RPI rows this instruction writes
+            const int r0 = frag_row(tm - 1) + pass * RPI;   // first of the RPI rows this instruction writes
             if (ALL_ROWS || r0 + RPI <= m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);   // wave-uniform test
-            else if (r0 + rd_row < m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);    // ragged last rows
+            else if (do_store && r0 + rd_row < m_rem) store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);    // ragged last rows
             dst += dst_step;
           }
           __builtin_amdgcn_sched_barrier(0);
         }
+        if (tm > 0 && TS::WM > 1) dst += frag_step;
         xsv = xsv_next;
       }
     } else {
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) {
+        if (tm >= fm_live) continue;   // no valid row in this fragment (wave-uniform)
         park(tm, 0, TS::FN, xs_lds[tm * 16 + j]);
         uint4 vals[NP];
         fetch(tm, vals);
 #pragma unroll
         for (int pass = 0; pass < NP; ++pass) {
           const uint4 val = vals[pass];
-          const int mm = m_base + tm * 16 + pass * RPI + rd_row;
+          const int mm = frag_row(tm) + pass * RPI + rd_row;
           const int nn = n_base + rd_chunk * 8;
           uint16_t* dst = dst_of(tm, pass);
           if (mm >= m_rem || nn >= n_rem) continue;

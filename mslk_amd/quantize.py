@@ -1,8 +1,9 @@
 """Row-wise FP8 quantization behind the reference's Python interface.
 
-`quantize_fp8_row` keeps the signature of the reference function
-(mslk/quantize/triton/fp8_quantize.py:319-328) and produces, on the GPU, the bits of its torch
-branch (356-378).  `quantize_fp8_per_row` is the legacy operator name for the same computation.
+`quantize_fp8_row` keeps the signature, the operator name (`triton::quantize_fp8_row`) and the dispatch of the
+reference function (mslk/quantize/triton/fp8_quantize.py:319-378): `use_triton=True` selects the arithmetic of its
+GPU kernel, `use_triton=False` the bits of its torch emulation (356-378).  `quantize_fp8_per_row`
+(`mslk::quantize_fp8_per_row`) always gives the latter.
 """
 from __future__ import annotations
 
@@ -45,9 +46,10 @@ class _on_device:
             self.ctx.__exit__(*exc)
 
 
-def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, align_rows_to: Optional[int] = None,
-                   zero_start_index_M: Optional[torch.Tensor] = None, triton_eps: Optional[float] = None
-                   ) -> Tuple[torch.Tensor, torch.Tensor]:
+def _quantize_launch(a: torch.Tensor, scale_ub: Optional[torch.Tensor], zero_start_index_M: Optional[torch.Tensor],
+                     align_rows_to: Optional[int], triton_eps: Optional[float]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One quantizer launch.  `triton_eps` None: the arithmetic of the reference's torch branch; a float: the arithmetic of
+    its Triton kernel with that lower bound of amax."""
     if a.dtype not in _DTYPE_CODE:
         raise RuntimeError(f"quantize_fp8_row: unsupported input dtype {a.dtype} (bf16, fp16, fp32 are supported)")
     if a.dim() < 1:
@@ -76,7 +78,9 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
     scale = torch.empty(lead, dtype=torch.float32, device=a.device)
     ub_ptr = None
     if scale_ub is not None:
-        scale_ub = scale_ub.to(device=a.device, dtype=torch.float32).reshape(-1)[:1].contiguous()
+        if scale_ub.device != a.device:
+            raise RuntimeError("'scale_ub' must be on the same device as 'a'")   # fp8_quantize.py:229-230
+        scale_ub = scale_ub.to(dtype=torch.float32).reshape(-1)[:1].contiguous()
         ub_ptr = scale_ub.data_ptr()
     zs_ptr, zs_code, rows_per_group = None, 0, 1
     if zero_start_index_M is not None:
@@ -94,60 +98,99 @@ def _quantize_impl(a: torch.Tensor, scale_ub: Optional[torch.Tensor] = None, ali
         zs_ptr, zs_code = zs.data_ptr(), (0 if zs.dtype == torch.int64 else 1)
     if rows == 0:
         return xq, scale
-    if triton_eps is not None:
-        # arithmetic of the reference's Triton kernel (fp8_quantize.py:131-207) instead of its torch branch
-        with _on_device(a.device):
+    with _on_device(a.device):
+        if triton_eps is not None:
             _lib.check(_lib.lib().mslk_amd_quantize_fp8_row_triton_arithmetic(
                 a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out, scale.data_ptr(), ub_ptr,
                 float(triton_eps), zs_ptr, zs_code, rows_per_group, _stream_ptr(a.device)))
-        return xq, scale
-    if zs_ptr is not None:
-        with _on_device(a.device):
+        elif zs_ptr is not None:
             _lib.check(_lib.lib().mslk_amd_quantize_fp8_row_jagged(
                 a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
                 scale.data_ptr(), ub_ptr, zs_ptr, zs_code, rows_per_group, _stream_ptr(a.device)))
-        return xq, scale
-    if rows > 0:
-        with _on_device(a.device):
+        else:
             _lib.check(_lib.lib().mslk_amd_quantize_fp8_row(
                 a2.data_ptr(), _DTYPE_CODE[a.dtype], rows, K, row_stride, xq.data_ptr(), K_out,
                 scale.data_ptr(), ub_ptr, _stream_ptr(a.device)))
     return xq, scale
 
 
-def _quantize_fp8_row_fake(a, scale_ub=None, align_rows_to=None, zero_start_index_M=None, triton_eps=None):
+# Lower bound of amax when the caller passes eps_opt=None: get_fp8_constants()'s eps (mslk/utils/triton/fp8_utils.py:23-40).
+_FP8_EPS = 1e-12
+
+
+def _quantize_fp8_row_gpu(a, scale_ub=None, zero_start_index_M=None, use_triton=True, output_device=None,
+                          align_rows_to=None, eps_opt=1.0 / 512.0):
+    """GPU kernel of `triton::quantize_fp8_row` (reference: fp8_quantize.py:319-378).  As in the reference, `use_triton`
+    picks the arithmetic: True = its GPU (Triton) kernel's -- amax clamped at `eps_opt`, scale = amax / 448,
+    code = clamp(x / scale, +-448), saturating (131-207) -- False = its torch branch's -- amax clamped at 1e-12 in the input
+    dtype, inv = (1 / amax) * 448, code = cast(x * inv) without saturation, scale = 1 / inv (356-378).  The torch branch of
+    the reference ignores `zero_start_index_M` and `align_rows_to`; here both arithmetics honour them."""
+    triton_eps = None
+    if use_triton:
+        triton_eps = eps_opt if eps_opt is not None else _FP8_EPS
+    a_fp8, a_scale = _quantize_launch(a, scale_ub, zero_start_index_M, align_rows_to, triton_eps)
+    if output_device is not None and torch.device(output_device) != a.device:
+        a_fp8, a_scale = a_fp8.to(output_device), a_scale.to(output_device)
+    return a_fp8, a_scale
+
+
+def _quantize_fp8_row_fake(a, scale_ub=None, zero_start_index_M=None, use_triton=True, output_device=None,
+                           align_rows_to=None, eps_opt=1.0 / 512.0):
     # shape function of the reference (fp8_quantize.py:381-407)
+    dev = a.device if output_device is None else output_device
     K = a.shape[-1]
     if align_rows_to is not None:
         K = (K + align_rows_to - 1) // align_rows_to * align_rows_to
-    return (torch.empty(tuple(a.shape[:-1]) + (K,), dtype=FP8_DTYPE, device=a.device),
-            torch.empty(a.shape[:-1], dtype=torch.float32, device=a.device))
+    return (torch.empty(tuple(a.shape[:-1]) + (K,), dtype=FP8_DTYPE, device=dev),
+            torch.empty(a.shape[:-1], dtype=torch.float32, device=dev))
 
 
-# Registered with the low-level library API (a few microseconds of dispatch per call); GPU kernel only.
+def _quantize_fp8_per_row_gpu(input, bs=None, scale_ub=None, output_dtype=None, stochastic_rounding=False):
+    """GPU kernel of `mslk::quantize_fp8_per_row`: row amax, scale = amax / 448, cast to e4m3fn, with the bits of the
+    reference's torch emulation (fp8_quantize.py:356-378)."""
+    if bs is not None:
+        raise NotImplementedError("quantize_fp8_per_row: `bs` is not supported")
+    if stochastic_rounding:
+        raise NotImplementedError("quantize_fp8_per_row: stochastic rounding is not supported")
+    if output_dtype is not None and output_dtype != FP8_DTYPE:
+        raise RuntimeError(f"quantize_fp8_per_row: only {FP8_DTYPE} output is supported on gfx950")
+    return _quantize_launch(input, scale_ub, None, None, None)
+
+
+def _quantize_fp8_per_row_fake(input, bs=None, scale_ub=None, output_dtype=None, stochastic_rounding=False):
+    return (torch.empty(input.shape, dtype=FP8_DTYPE, device=input.device),
+            torch.empty(input.shape[:-1], dtype=torch.float32, device=input.device))
+
+
+# Registered with the low-level library API (a few microseconds of dispatch per call); GPU kernels only.  The names and
+# schemas are the ones callers of the reference use: `triton::quantize_fp8_row` is what its
+# torch.library.custom_op (fp8_quantize.py:319-328) defines, so a traced or compiled caller of
+# torch.ops.triton.quantize_fp8_row lands here; when the reference defined the op first only its GPU kernel is replaced.
 _library = torch.library.Library("mslk", "FRAGMENT")
-if not hasattr(torch.ops.mslk, "quantize_fp8_row"):
-    _library.define("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, int? align_rows_to=None, "
-                    "Tensor? zero_start_index_M=None, float? triton_eps=None) -> (Tensor, Tensor)")
-    _library.impl("quantize_fp8_row", _quantize_impl, "CUDA")
-    torch.library.register_fake("mslk::quantize_fp8_row", _quantize_fp8_row_fake, lib=_library)
+_triton_library = torch.library.Library("triton", "FRAGMENT")
+_QUANTIZE_ROW_SCHEMA = ("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, Tensor? zero_start_index_M=None, "
+                        "bool use_triton=True, Device? output_device=None, SymInt? align_rows_to=None, "
+                        "float? eps_opt=0.001953125) -> (Tensor, Tensor)")
+_QUANTIZE_PER_ROW_SCHEMA = ("quantize_fp8_per_row(Tensor input, Tensor? bs=None, Tensor? scale_ub=None, "
+                            "ScalarType? output_dtype=None, bool stochastic_rounding=False) -> (Tensor, Tensor)")
 
 
-_NUMERICS = "torch"
+def _register_quantize() -> None:
+    if hasattr(torch.ops.triton, "quantize_fp8_row"):
+        _triton_library.impl("quantize_fp8_row", _quantize_fp8_row_gpu, "CUDA", allow_override=True)
+    else:
+        _triton_library.define(_QUANTIZE_ROW_SCHEMA)
+        _triton_library.impl("quantize_fp8_row", _quantize_fp8_row_gpu, "CUDA")
+        torch.library.register_fake("triton::quantize_fp8_row", _quantize_fp8_row_fake, lib=_triton_library)
+    if hasattr(torch.ops.mslk, "quantize_fp8_per_row"):
+        _library.impl("quantize_fp8_per_row", _quantize_fp8_per_row_gpu, "CUDA", allow_override=True)
+    else:
+        _library.define(_QUANTIZE_PER_ROW_SCHEMA)
+        _library.impl("quantize_fp8_per_row", _quantize_fp8_per_row_gpu, "CUDA")
+        torch.library.register_fake("mslk::quantize_fp8_per_row", _quantize_fp8_per_row_fake, lib=_library)
 
 
-def set_quantize_numerics(which: str) -> None:
-    """Which of the reference's two arithmetics `quantize_fp8_row` reproduces.
-
-    "torch" (default): the torch branch (fp8_quantize.py:356-378) for every call -- the bit contract this
-    package is tested against.  "triton": calls with `use_triton=True` use the arithmetic of the reference's
-    Triton kernel (fp8_quantize.py:131-207: amax clamped at `eps_opt`, scale = amax / 448, code =
-    clamp(x / scale, +-448) with IEEE divisions), as the reference does for GPU tensors; `use_triton=False`
-    still selects the torch branch."""
-    global _NUMERICS
-    if which not in ("torch", "triton"):
-        raise ValueError("quantize numerics must be 'torch' or 'triton'")
-    _NUMERICS = which
+_register_quantize()
 
 
 def quantize_fp8_row(
@@ -159,27 +202,22 @@ def quantize_fp8_row(
     align_rows_to: Optional[int] = None,
     eps_opt: Optional[float] = 1.0 / 512.0,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Quantize `a` to e4m3fn with one fp32 scale per row (reference signature, fp8_quantize.py:320-343).
+    """Quantize `a` to e4m3fn with one fp32 scale per row (reference signature and dispatch, fp8_quantize.py:319-378).
 
     Returns (a_fp8 with a's shape [last dim padded to align_rows_to], scale with shape a.shape[:-1]).
-    The numerics are those of the reference's torch branch (the contract this build is checked
-    against bit for bit): amax is clamped at 1e-12 in the input dtype, so `eps_opt` -- which only the
-    reference's Triton branch reads -- has no effect, and `use_triton` is ignored, unless
-    `set_quantize_numerics("triton")` was called (then `use_triton=True` selects the Triton kernel's arithmetic
-    with `eps_opt`, as the reference does on a GPU).  With `zero_start_index_M` (one entry per [N, K] matrix of the input viewed as
-    [B, M, N, K]) the rows n >= zero_start_index_M[b, m] are not read and quantize like all-zero rows
-    (fp8_quantize.py:123-129).
+    `use_triton=True` (the default, as in the reference) gives the arithmetic of the reference's GPU kernel: amax
+    clamped at `eps_opt` (and `scale_ub`), scale = amax / 448, codes = clamp(a / scale, +-448).  `use_triton=False` gives
+    the bits of the reference's torch emulation -- the contract this build is checked against bit for bit: amax clamped
+    at 1e-12 in the input dtype, inv = (1 / amax) * 448, codes = cast(a * inv) (values beyond 464 become NaN codes,
+    which only happens when `scale_ub` cuts the row maximum), scale = 1 / inv; `eps_opt` has no effect there.
+    With `zero_start_index_M` (one entry per [N, K] matrix of the input viewed as [B, M, N, K]) the rows
+    n >= zero_start_index_M[b, m] are not read and quantize like all-zero rows (fp8_quantize.py:123-129).
     The input must live on a GPU: there is no CPU implementation in this package.
     """
     if not a.is_cuda:
         raise RuntimeError("mslk_amd.quantize_fp8_row: input must be a GPU tensor (no CPU implementation)")
-    triton_eps = None
-    if _NUMERICS == "triton" and use_triton:
-        triton_eps = eps_opt if eps_opt is not None else 1e-12   # get_fp8_constants() eps (fp8_quantize.py:243-247)
-    a_fp8, a_scale = torch.ops.mslk.quantize_fp8_row(a, scale_ub, align_rows_to, zero_start_index_M, triton_eps)
-    if output_device is not None and torch.device(output_device) != a.device:
-        a_fp8, a_scale = a_fp8.to(output_device), a_scale.to(output_device)
-    return a_fp8, a_scale
+    return torch.ops.triton.quantize_fp8_row(a, scale_ub, zero_start_index_M, use_triton, output_device, align_rows_to,
+                                             eps_opt)
 
 
 def _dequantize_impl(xq: torch.Tensor, x_scale: torch.Tensor) -> torch.Tensor:
@@ -226,13 +264,10 @@ def quantize_fp8_per_row(
     output_dtype: Optional[torch.dtype] = None,
     stochastic_rounding: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Legacy operator name for the same row-wise quantization (the reference's bench still calls the
-    path `CudaFP8Rowwise`, bench/quantize/quantize_ops.py:242-251).  `bs` and stochastic rounding
-    are not supported."""
-    if bs is not None:
-        raise NotImplementedError("quantize_fp8_per_row: `bs` is not supported")
-    if stochastic_rounding:
-        raise NotImplementedError("quantize_fp8_per_row: stochastic rounding is not supported")
-    if output_dtype is not None and output_dtype != FP8_DTYPE:
-        raise RuntimeError(f"quantize_fp8_per_row: only {FP8_DTYPE} output is supported on gfx950")
-    return quantize_fp8_row(input, scale_ub=scale_ub)
+    """Row amax -> scale = amax / 448 -> e4m3fn codes, bit-exact to the reference's torch emulation
+    (`quantize_fp8_row(..., use_triton=False)`, fp8_quantize.py:356-378); the legacy operator name of the path (the
+    reference's bench still calls it `CudaFP8Rowwise`, bench/quantize/quantize_ops.py:242-251).  `bs` and stochastic
+    rounding are not supported."""
+    if not input.is_cuda:
+        raise RuntimeError("mslk_amd.quantize_fp8_per_row: input must be a GPU tensor (no CPU implementation)")
+    return torch.ops.mslk.quantize_fp8_per_row(input, bs, scale_ub, output_dtype, stochastic_rounding)

@@ -73,7 +73,15 @@ def test_ops_registered_with_reference_schemas():
                  "Tensor? bias=None, bool use_fast_accum=True) -> Tensor")
     s = str(torch.ops.mslk.f8f8bf16_rowwise_grouped_dynamic.default._schema)
     assert s.endswith("Tensor zero_start_index_M, bool zeroing_output_tensor=True) -> Tensor")
-    assert hasattr(torch.ops.mslk, "quantize_fp8_row") and hasattr(torch.ops.mslk, "dequantize_fp8_row")
+    assert hasattr(torch.ops.mslk, "dequantize_fp8_row")
+    # the quantizer under the names callers of the reference use (mslk/quantize/triton/fp8_quantize.py:319-328)
+    s = str(torch.ops.triton.quantize_fp8_row.default._schema)
+    assert s == ("triton::quantize_fp8_row(Tensor a, Tensor? scale_ub=None, Tensor? zero_start_index_M=None, "
+                 "bool use_triton=True, Device? output_device=None, SymInt? align_rows_to=None, "
+                 "float? eps_opt=0.001953125) -> (Tensor, Tensor)")
+    s = str(torch.ops.mslk.quantize_fp8_per_row.default._schema)
+    assert s == ("mslk::quantize_fp8_per_row(Tensor input, Tensor? bs=None, Tensor? scale_ub=None, "
+                 "ScalarType? output_dtype=None, bool stochastic_rounding=False) -> (Tensor, Tensor)")
 
 
 def test_fake_kernels_give_reference_shapes():
@@ -105,8 +113,10 @@ def test_fake_kernels_give_reference_shapes():
             torch.empty(3, 40, 512, dtype=F8, device=dev), torch.empty(3, 768, 512, dtype=F8, device=dev),
             torch.empty(3, 40, device=dev), torch.empty(3, 768, device=dev))
         assert y.shape == (3, 40, 768) and y.dtype == torch.bfloat16
-        q, s = torch.ops.mslk.quantize_fp8_row(torch.empty(2, 3, 100, dtype=torch.bfloat16, device=dev), None, 16)
+        q, s = torch.ops.triton.quantize_fp8_row(torch.empty(2, 3, 100, dtype=torch.bfloat16, device=dev), align_rows_to=16)
         assert q.shape == (2, 3, 112) and q.dtype == F8 and s.shape == (2, 3) and s.dtype == torch.float32
+        q, s = torch.ops.mslk.quantize_fp8_per_row(torch.empty(5, 100, dtype=torch.float16, device=dev))
+        assert q.shape == (5, 100) and q.dtype == F8 and s.shape == (5,) and s.dtype == torch.float32
 
 
 def test_argument_checks_raise_like_the_reference():

@@ -198,7 +198,7 @@ def test_hip_graph_capture_and_replay(M, N, K):
     g = torch.Generator().manual_seed(24)
     xq, wq, xs, ws = _gpu(*_random_problem(M, N, K, g))
     x_bf16 = torch.randn(M, K, device=DEV).bfloat16()
-    eager_q, eager_s = mslk_amd.quantize_fp8_row(x_bf16)
+    eager_q, eager_s = mslk_amd.quantize_fp8_row(x_bf16, use_triton=False)
     eager = torch.ops.mslk.f8f8bf16_rowwise(eager_q, wq, eager_s, ws)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
@@ -206,11 +206,11 @@ def test_hip_graph_capture_and_replay(M, N, K):
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         for _ in range(2):
-            q, s = mslk_amd.quantize_fp8_row(x_bf16)
+            q, s = mslk_amd.quantize_fp8_row(x_bf16, use_triton=False)
             torch.ops.mslk.f8f8bf16_rowwise(q, wq, s, ws)
     torch.cuda.current_stream().wait_stream(side)
     with torch.cuda.graph(graph):
-        q, s = mslk_amd.quantize_fp8_row(x_bf16)
+        q, s = mslk_amd.quantize_fp8_row(x_bf16, use_triton=False)
         y = torch.ops.mslk.f8f8bf16_rowwise(q, wq, s, ws)
     for _ in range(3):
         y.fill_(0)
@@ -232,7 +232,7 @@ def _check_sampled(y, xq, wq, xs, ws, bias, g, rows=48, what=""):
 
 def _quantize_gpu_checked(t_cpu, g, rows=32):
     """Quantize on the GPU and confirm a sample of rows bit-exact against the oracle."""
-    q, s = mslk_amd.quantize_fp8_row(t_cpu.to(DEV))
+    q, s = mslk_amd.quantize_fp8_row(t_cpu.to(DEV), use_triton=False)
     idx = torch.randperm(t_cpu.shape[0], generator=g)[: min(rows, t_cpu.shape[0])]
     rq, rs = O.quantize_fp8_row(t_cpu[idx])
     assert torch.equal(q[idx.to(DEV)].cpu().view(torch.uint8), rq.view(torch.uint8))
@@ -244,7 +244,7 @@ def test_cfg0_full():
     wl = W.cfg0()
     xq, xs = _quant_cpu(wl.x)
     wq, ws = _quant_cpu(wl.w)
-    gq, gs = mslk_amd.quantize_fp8_row(wl.x.to(DEV))
+    gq, gs = mslk_amd.quantize_fp8_row(wl.x.to(DEV), use_triton=False)
     assert torch.equal(gq.cpu().view(torch.uint8), xq.view(torch.uint8)) and torch.equal(gs.cpu().view(torch.int32), xs.view(torch.int32))
     y = _op(xq, wq, xs, ws)
     assert_gemm_close(y, O.dequant_matmul(xq, wq, xs, ws), "cfg0")
@@ -290,7 +290,7 @@ def test_cfg3_decode(M):
     w = W.cfg3_weight()
     wq, ws = _quantize_gpu_checked(w, g)
     x = W.cfg3_activations(M)
-    xq, xs = mslk_amd.quantize_fp8_row(x.to(DEV))
+    xq, xs = mslk_amd.quantize_fp8_row(x.to(DEV), use_triton=False)
     rq, rs = O.quantize_fp8_row(x)
     assert torch.equal(xq.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs.cpu().view(torch.int32), rs.view(torch.int32))
     y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)

@@ -97,7 +97,7 @@ def test_quantize_beyond_2_32_elements():
     rows, K = 66000, 65536 + 8                   # 4.33e9 elements: codes cross 2^32 bytes at row 65528, input at 32764
     g = torch.Generator(device=DEV).manual_seed(9)
     x = torch.randn(rows, K, device=DEV, dtype=torch.bfloat16, generator=g)
-    xq, scale = mslk_amd.quantize_fp8_row(x)
+    xq, scale = mslk_amd.quantize_fp8_row(x, use_triton=False)
     torch.cuda.synchronize()
     picks = torch.cat([_rows_around(2**32 // K, rows - 1), _rows_around(2**31 // K, rows - 1),
                        _rows_around(2**30 // K, rows - 1)]).unique()

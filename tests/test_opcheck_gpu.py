@@ -19,9 +19,11 @@ def _codes(*shape):
 
 def test_opcheck_quantize_and_dequantize():
     x = torch.randn(48, 256, device=DEV, dtype=torch.bfloat16)
-    torch.library.opcheck(torch.ops.mslk.quantize_fp8_row, (x,), test_utils=CHECKS)
-    torch.library.opcheck(torch.ops.mslk.quantize_fp8_row, (x, torch.tensor([1200.0], device=DEV), 64), test_utils=CHECKS)
-    q, s = torch.ops.mslk.quantize_fp8_row(x)
+    torch.library.opcheck(torch.ops.triton.quantize_fp8_row, (x,), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.mslk.quantize_fp8_per_row, (x,), test_utils=CHECKS)
+    torch.library.opcheck(torch.ops.triton.quantize_fp8_row, (x, torch.tensor([1200.0], device=DEV), None, False, None, 64),
+                          test_utils=CHECKS)
+    q, s = torch.ops.triton.quantize_fp8_row(x)
     torch.library.opcheck(torch.ops.mslk.dequantize_fp8_row, (q, s), test_utils=CHECKS)
 
 
@@ -95,7 +97,7 @@ def test_ops_trace_under_torch_compile():
     wq, ws = mslk_amd.quantize_fp8_row(w)
 
     def linear(x):
-        xq, xs = torch.ops.mslk.quantize_fp8_row(x)
+        xq, xs = torch.ops.triton.quantize_fp8_row(x)
         return torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
 
     x = torch.randn(40, 256, device=DEV, dtype=torch.bfloat16)

@@ -17,7 +17,7 @@ ALL_BF16 = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfl
 
 def _run(a_cpu, scale_ub=None, align=None):
     ub = None if scale_ub is None else scale_ub.to(DEV)
-    xq, s = mslk_amd.quantize_fp8_row(a_cpu.to(DEV), scale_ub=ub, align_rows_to=align)
+    xq, s = mslk_amd.quantize_fp8_row(a_cpu.to(DEV), scale_ub=ub, align_rows_to=align, use_triton=False)
     torch.cuda.synchronize()
     return xq, s
 
@@ -98,7 +98,7 @@ def test_many_short_rows(dtype):
         assert_quant_bit_exact(a, xq, s, K_out=112)
     b = torch.randn(8, 600, 128, generator=g).to(dtype)          # 4800 rows in 8 groups, some rows dead
     zs = torch.tensor([600, 0, 1, 599, 300, 17, 600, 64], dtype=torch.int64)
-    xq, s = mslk_amd.quantize_fp8_row(b.to(DEV), zero_start_index_M=zs.to(DEV))
+    xq, s = mslk_amd.quantize_fp8_row(b.to(DEV), zero_start_index_M=zs.to(DEV), use_triton=False)
     torch.cuda.synchronize()
     rq, rs = O.quantize_fp8_row_jagged(b, zs)
     assert torch.equal(codes(xq), codes(rq)) and torch.equal(bits32(s), bits32(rs))
@@ -201,7 +201,8 @@ def test_jagged_rows(shape, align, idx_dtype):
     poisoned = a.clone().view(groups, shape[-2], shape[-1])
     for gi in range(groups):
         poisoned[gi, int(zs[gi]):] = float("nan")
-    xq, s = mslk_amd.quantize_fp8_row(poisoned.view(shape).to(DEV), zero_start_index_M=zs.to(DEV), align_rows_to=align)
+    xq, s = mslk_amd.quantize_fp8_row(poisoned.view(shape).to(DEV), zero_start_index_M=zs.to(DEV), align_rows_to=align,
+                                       use_triton=False)
     torch.cuda.synchronize()
     rq, rs = O.quantize_fp8_row_jagged(a, zs)
     K = shape[-1]
@@ -240,51 +241,59 @@ def test_dequantize_bit_exact(shape):
 def test_dequantize_round_trip_full_size():
     g = torch.Generator().manual_seed(12)
     a = torch.randn(4096, 4096, generator=g).bfloat16().to(DEV)
-    xq, s = mslk_amd.quantize_fp8_row(a)
+    xq, s = mslk_amd.quantize_fp8_row(a, use_triton=False)
     back = mslk_amd.dequantize_fp8_row(xq, s).float()
     af = a.float()
     assert ((back - af).abs() <= af.abs() * 2.0 ** -4 + af.abs().amax(dim=1, keepdim=True) * 2.0 ** -9).all()
     # dequantize(quantize(.)) is idempotent: quantizing the result again reproduces codes and values
-    xq2, s2 = mslk_amd.quantize_fp8_row(back.bfloat16())
+    xq2, s2 = mslk_amd.quantize_fp8_row(back.bfloat16(), use_triton=False)
     back2 = mslk_amd.dequantize_fp8_row(xq2, s2).float()
     assert (back2 - back).abs().max() <= back.abs().max() * 2.0 ** -7
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_triton_arithmetic_mode(dtype):
-    """`set_quantize_numerics("triton")`: codes and scales equal the oracle's restatement of the reference's
-    Triton kernel bit for bit (IEEE divisions on both sides), over the reference's shape sweep, eps variants,
-    scale_ub, jagged rows and padding; the default mode is unaffected."""
+    """`use_triton=True` (the default, as in the reference): codes and scales equal the oracle's restatement of the
+    reference's Triton kernel bit for bit (IEEE divisions on both sides), over the reference's shape sweep, eps variants,
+    scale_ub, jagged rows and padding; `use_triton=False` gives the torch emulation."""
     g = torch.Generator().manual_seed(17)
-    mslk_amd.set_quantize_numerics("triton")
-    try:
-        for shape in [(1, 16), (7, 777), (64, 1024), (2500, 4096), (3, 5, 136), (5, 20000)]:
-            a = (torch.randn(shape, generator=g) * 3).to(dtype)
-            a.view(-1, shape[-1])[0].zero_()                        # a zero row: the eps clamp decides
-            a.view(-1, shape[-1])[-1].mul_(2.0 ** -14)               # a row below 1/512
-            for eps_opt, ub in [(1.0 / 512.0, None), (None, None), (1e-4, 1.2345), (1.0 / 512.0, 1200.0)]:
-                ubt = None if ub is None else torch.tensor([ub], dtype=torch.float32)
-                xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), scale_ub=None if ubt is None else ubt.to(DEV), eps_opt=eps_opt)
-                torch.cuda.synchronize()
-                rq, rs = O.quantize_fp8_row_triton_arithmetic(a, ubt, eps_opt if eps_opt is not None else 1e-12)
-                assert torch.equal(codes(xq), codes(rq)), (shape, eps_opt, ub)
-                assert torch.equal(bits32(s), bits32(rs)), (shape, eps_opt, ub)
-        # use_triton=False keeps the torch branch
-        a = torch.randn(33, 256, generator=g).to(dtype)
-        xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), use_triton=False)
-        assert_quant_bit_exact(a, xq, s)
-        # jagged + padding
-        a = torch.randn(4, 6, 40, generator=g).to(dtype)
-        zs = torch.tensor([6, 0, 3, 1])
-        xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=zs.to(DEV), align_rows_to=16)
-        masked = a.clone()
-        for gi in range(4):
-            masked[gi, int(zs[gi]):] = 0
-        rq, rs = O.quantize_fp8_row_triton_arithmetic(masked)
-        assert torch.equal(codes(xq)[..., :40], codes(rq)) and (codes(xq)[..., 40:] == 0).all()
-        assert torch.equal(bits32(s), bits32(rs))
-    finally:
-        mslk_amd.set_quantize_numerics("torch")
-    a = torch.randn(8, 64, generator=g).to(dtype)
-    xq, s = mslk_amd.quantize_fp8_row(a.to(DEV))
+    for shape in [(1, 16), (7, 777), (64, 1024), (2500, 4096), (3, 5, 136), (5, 20000)]:
+        a = (torch.randn(shape, generator=g) * 3).to(dtype)
+        a.view(-1, shape[-1])[0].zero_()                        # a zero row: the eps clamp decides
+        a.view(-1, shape[-1])[-1].mul_(2.0 ** -14)               # a row below 1/512
+        for eps_opt, ub in [(1.0 / 512.0, None), (None, None), (1e-4, 1.2345), (1.0 / 512.0, 1200.0)]:
+            ubt = None if ub is None else torch.tensor([ub], dtype=torch.float32)
+            xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), scale_ub=None if ubt is None else ubt.to(DEV), eps_opt=eps_opt)
+            torch.cuda.synchronize()
+            rq, rs = O.quantize_fp8_row_triton_arithmetic(a, ubt, eps_opt if eps_opt is not None else 1e-12)
+            assert torch.equal(codes(xq), codes(rq)), (shape, eps_opt, ub)
+            assert torch.equal(bits32(s), bits32(rs)), (shape, eps_opt, ub)
+    # use_triton=False selects the torch branch, and so does the legacy operator
+    a = torch.randn(33, 256, generator=g).to(dtype)
+    xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), use_triton=False)
     assert_quant_bit_exact(a, xq, s)
+    xq, s = torch.ops.mslk.quantize_fp8_per_row(a.to(DEV))
+    assert_quant_bit_exact(a, xq, s)
+    # jagged + padding
+    a = torch.randn(4, 6, 40, generator=g).to(dtype)
+    zs = torch.tensor([6, 0, 3, 1])
+    xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), zero_start_index_M=zs.to(DEV), align_rows_to=16)
+    masked = a.clone()
+    for gi in range(4):
+        masked[gi, int(zs[gi]):] = 0
+    rq, rs = O.quantize_fp8_row_triton_arithmetic(masked)
+    assert torch.equal(codes(xq)[..., :40], codes(rq)) and (codes(xq)[..., 40:] == 0).all()
+    assert torch.equal(bits32(s), bits32(rs))
+
+
+def test_default_arithmetic_saturates_under_scale_ub():
+    """A GPU caller of the reference gets its Triton kernel by default, which stores +-448 where `scale_ub` cuts the row
+    maximum (fp8_quantize.py:142-144,164-166); the torch emulation stores NaN codes there."""
+    a = torch.tensor([[1.0, -2.0, 1000.0, -3000.0] * 16], dtype=torch.bfloat16)
+    ub = torch.tensor([2.0], device=DEV)
+    xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), scale_ub=ub)
+    c = codes(xq)[0, :4].tolist()
+    assert c == [0x76, 0xFE, 0x7E, 0xFE], [hex(v) for v in c]     # 1 / (2 / 448) = 224, -448, +448 (saturated), -448
+    assert s.cpu().item() == (torch.tensor(2.0) / 448.0).item()    # fl32(2 / 448)
+    xq, s = mslk_amd.quantize_fp8_row(a.to(DEV), scale_ub=ub, use_triton=False)
+    assert (codes(xq)[0, 2:4] & 0x7F).tolist() == [0x7F, 0x7F]   # no saturation in the torch emulation
