@@ -55,6 +55,58 @@ def _events_ms(fn, iters):
     return start.elapsed_time(stop) / iters
 
 
+SETTLE_MS = 50.0
+
+
+def _settle(fn, min_ms=SETTLE_MS):
+    """Clock-settling phase OUTSIDE every timed region: fn(i) is launched until at least `min_ms` of GPU time has passed
+    (the shader clock, the power state and the caches reach the state a long-running job sees; a handful of warm-up
+    steps does not get there).  Returns the number of launches."""
+    import torch
+    start = torch.cuda.Event(enable_timing=True)
+    start.record()
+    n = 0
+    while True:
+        for _ in range(32):
+            fn(n)
+            n += 1
+        stop = torch.cuda.Event(enable_timing=True)
+        stop.record()
+        stop.synchronize()
+        if start.elapsed_time(stop) >= min_ms:
+            return n
+
+
+def _parity(y, xq, wq, xs, ws, bias=None, block=2048):
+    """The three accuracy figures of the path for one output, against the rowwise-dequantized fp32 product formed on the
+    GPU with plain torch (a floating-point reference, not the product path): max|y-ref|/max|ref|, ||y-ref||_F/||ref||_F and
+    the number of elements beyond |y-ref| <= 1e-2 |ref| + 1e-2 rms(ref) (the elementwise form of the reference's tests,
+    test/gemm/gemm_test.py:493-505)."""
+    import torch
+    wd = wq.float() * ws.float()[:, None]
+    M = xq.shape[0]
+    max_abs_ref = 0.0
+    max_abs_diff = 0.0
+    sq_ref = 0.0
+    sq_diff = 0.0
+    refs = []
+    for r0 in range(0, M, block):
+        ref = (xq[r0:r0 + block].float() * xs[r0:r0 + block].float()[:, None]) @ wd.t()
+        if bias is not None:
+            ref += bias.float()[None, :]
+        d = y[r0:r0 + block].float() - ref
+        max_abs_ref = max(max_abs_ref, ref.abs().max().item())
+        max_abs_diff = max(max_abs_diff, d.abs().max().item())
+        sq_ref += ref.double().pow(2).sum().item()
+        sq_diff += d.double().pow(2).sum().item()
+        refs.append((r0, ref.abs(), d.abs()))
+    n = float(M) * wq.shape[0]
+    rms = (sq_ref / n) ** 0.5
+    bad = sum(int((d > 1e-2 * a + 1e-2 * rms).sum().item()) for _, a, d in refs)
+    return {"max_rel": max_abs_diff / max_abs_ref if max_abs_ref else 0.0, "normwise": (sq_diff / sq_ref) ** 0.5 if sq_ref else 0.0,
+            "elementwise_violations": bad, "elements": int(n)}
+
+
 def _median_events_ms(fn, iters, repeats=5):
     xs = sorted(_events_ms(fn, iters) for _ in range(repeats))
     return xs[len(xs) // 2]
@@ -208,7 +260,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
-    ap.add_argument("--only", default="", help="helper: run only this piece (gemm|quantize|decode|traffic|vendor) and exit")
+    ap.add_argument("--only", default="",
+                    help="helper: run only this piece (gemm|gemm-timed|quantize|decode|cfg2|grouped|traffic|vendor) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -255,7 +308,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_each_way": 256 << 20, "gemm_launches": 12}))
         return
-    if args.only in ("", "gemm"):
+    settle_launches = 0
+    if args.only in ("", "gemm", "gemm-timed"):
+        settle_launches = _settle(gemm_step)      # outside the timed region, named in config.workload
         for i in range(args.warmup):
             gemm_step(i)
         torch.cuda.synchronize()
@@ -271,6 +326,10 @@ def main():
         kern_ms = ev_start.elapsed_time(ev_stop) / args.steps
         value = flops / (wall_ms * 1e-3) / 1e12
         achieved = flops / (kern_ms * 1e-3) / 1e12
+        if args.only == "gemm-timed":   # for profiling: settle + warm-up + timed launches of the one kernel, nothing else
+            print(json.dumps({"gemm_ms": kern_ms, "tflops": achieved, "settle_launches": settle_launches}))
+            return
+        extras["parity_cfg1"] = _parity(sets[0][4], xq0, wq0, xs0, ws0)
         graph_ms = _graph_ms(gemm_step, 120)
         extras["gemm_cfg1_graph_replay"] = {"ms": graph_ms, "TFLOPs": flops / (graph_ms * 1e-3) / 1e12,
                                             "frac_mfma": flops / (graph_ms * 1e-3) / PEAK_FP8_FLOPS,
@@ -307,7 +366,19 @@ def main():
         q_ms = _median_events_ms(quant_step, 50)
         q_bytes = 3.0 * M * K + 4.0 * M
         extras["quantize_cfg1"] = {"ms": q_ms, "GBps": q_bytes / (q_ms * 1e-3) / 1e9,
-                                   "frac_hbm": q_bytes / (q_ms * 1e-3) / PEAK_HBM_BPS, "bytes": q_bytes}
+                                   "frac_hbm": q_bytes / (q_ms * 1e-3) / PEAK_HBM_BPS, "bytes": q_bytes,
+                                   "note": "arithmetic of the reference's torch emulation (use_triton=False)"}
+
+        def quant_triton_step(i):   # the arithmetic a GPU caller of the reference gets by default (IEEE divisions, saturating)
+            api.check(api.L.mslk_amd_quantize_fp8_row_triton_arithmetic(
+                xsets[i % len(xsets)].data_ptr(), 0, M, K, K, xq_tmp.data_ptr(), K, xs_tmp.data_ptr(), None, 1.0 / 512.0,
+                None, 0, 1, api.stream))
+
+        for i in range(10):
+            quant_triton_step(i)
+        qt_ms = _median_events_ms(quant_triton_step, 50)
+        extras["quantize_cfg1_triton_arithmetic"] = {"ms": qt_ms, "GBps": q_bytes / (qt_ms * 1e-3) / 1e9,
+                                                     "frac_hbm": q_bytes / (qt_ms * 1e-3) / PEAK_HBM_BPS}
         # dequantize_fp8_row on the same shape: 1 B in + 2 B out per element, rotating over 10 code sets
         qsets = [torch.randint(0, 120, (M, K), dtype=torch.uint8, device=dev).view(torch.float8_e4m3fn) for _ in range(10)]
         dq_out = [torch.empty(M, K, dtype=torch.bfloat16, device=dev) for _ in range(4)]
@@ -394,10 +465,16 @@ def main():
                 api.quantize(xd, xq3, xs3)
                 api.gemm(xq3, wsets[i % len(wsets)], xs3, ws3, y3)
 
+            def dec_fused_step(i):
+                api.check(api.L.mslk_amd_quantize_f8f8bf16_rowwise(xd.data_ptr(), 0, Kd, wsets[i % len(wsets)].data_ptr(),
+                                                                   ws3.data_ptr(), None, 0, y3.data_ptr(), Md, Nd, Kd,
+                                                                   None, None, api.stream))
+
             def dec_ps_step(i):
                 api.check(api.L.mslk_amd_f8f8_rowwise_preshuffle(xq3.data_ptr(), wshuf[i % len(wshuf)].data_ptr(), xs3.data_ptr(),
                                                                  ws3.data_ptr(), None, 0, y3.data_ptr(), 0, Md, Nd, Kd, api.stream))
 
+            _settle(dec_step, 20.0)
             for i in range(12):
                 dec_step(i)
                 dec_ps_step(i)
@@ -406,11 +483,24 @@ def main():
             ms_path = _median_events_ms(dec_path_step, 60)
             ms_graph = _graph_ms(dec_step, 60)
             nbytes = Nd * Kd + Md * Kd + 2.0 * Md * Nd + 4.0 * (Md + Nd)
+            fused = {}
+            if api.L.mslk_amd_quantize_f8f8bf16_rowwise_supported(Md, Nd, Kd):
+                for i in range(12):
+                    dec_fused_step(i)
+                ms_fused = _median_events_ms(dec_fused_step, 60)
+                fbytes = Nd * Kd + 2.0 * Md * Kd + 2.0 * Md * Nd + 4.0 * Nd      # bf16 activations in, no codes or scales in HBM
+                y1, q1, s1 = mslk_amd.quantize_f8f8bf16_rowwise(xd, wsets[0], ws3)
+                fused = {"ms_fused_quantize": ms_fused, "GBps_fused_quantize": fbytes / (ms_fused * 1e-3) / 1e9,
+                         "frac_hbm_fused_quantize": fbytes / (ms_fused * 1e-3) / PEAK_HBM_BPS,
+                         "fused_codes_and_scales_equal_quantizer": bool(torch.equal(q1.view(torch.uint8), xq3.view(torch.uint8))
+                                                                        and torch.equal(s1, xs3))}
+            dec_step(0)
+            par = _parity(y3, xq3, wsets[0], xs3, ws3)
             decode[f"M{Md}"] = {"ms": ms, "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm": nbytes / (ms * 1e-3) / PEAK_HBM_BPS,
                                 "ms_with_quantize": ms_path, "bytes": nbytes, "ms_graph_replay": ms_graph,
                                 "GBps_graph_replay": nbytes / (ms_graph * 1e-3) / 1e9,
                                 "ms_preshuffled_weights": ms_ps, "GBps_preshuffled_weights": nbytes / (ms_ps * 1e-3) / 1e9,
-                                "frac_hbm_preshuffled_weights": nbytes / (ms_ps * 1e-3) / PEAK_HBM_BPS}
+                                "frac_hbm_preshuffled_weights": nbytes / (ms_ps * 1e-3) / PEAK_HBM_BPS, **fused, "parity": par}
         extras["decode_N8192_K8192"] = decode
         del wsets, wshuf
         if args.only == "decode":
@@ -418,26 +508,33 @@ def main():
             return
 
     # ---------------------------------------------------------------- other configs (GEMM rate only)
-    if not args.no_extras:
+    if not args.no_extras and args.only == "":
         wl0 = W.cfg0()
         a, sa = mslk_amd.quantize_fp8_row(wl0.x.to(dev), use_triton=False)
         b, sb = mslk_amd.quantize_fp8_row(wl0.w.to(dev), use_triton=False)
         y0 = torch.empty(1024, 1024, dtype=torch.bfloat16, device=dev)
         ms = _median_events_ms(lambda i: api.gemm(a, b, sa, sb, y0), 100)
-        extras["gemm_cfg0_1024"] = {"ms": ms, "TFLOPs": 2.0 * 1024**3 / (ms * 1e-3) / 1e12}
+        extras["gemm_cfg0_1024"] = {"ms": ms, "TFLOPs": 2.0 * 1024**3 / (ms * 1e-3) / 1e12, "parity": _parity(y0, a, b, sa, sb)}
+
+    if (not args.no_extras and args.only == "") or args.only == "cfg2":
 
         wl2 = W.cfg2()
         a, sa = mslk_amd.quantize_fp8_row(wl2.x.to(dev), use_triton=False)
         b, sb = mslk_amd.quantize_fp8_row(wl2.w.to(dev), use_triton=False)
         bias2 = wl2.bias.to(dev)
         y2 = torch.empty(8192, 28672, dtype=torch.bfloat16, device=dev)
-        for _ in range(30):
-            api.gemm(a, b, sa, sb, y2, bias2)
+        _settle(lambda i: api.gemm(a, b, sa, sb, y2, bias2))
         ms = _median_events_ms(lambda i: api.gemm(a, b, sa, sb, y2, bias2), 10)
         f2 = 2.0 * 8192 * 28672 * 4096
         extras["gemm_cfg2_8192x28672x4096_bias"] = {"ms": ms, "TFLOPs": f2 / (ms * 1e-3) / 1e12,
-                                                     "frac_mfma": f2 / (ms * 1e-3) / PEAK_FP8_FLOPS}
+                                                     "frac_mfma": f2 / (ms * 1e-3) / PEAK_FP8_FLOPS,
+                                                     "parity": _parity(y2, a, b, sa, sb, bias2)}
         del a, b, y2, wl2
+        if args.only == "cfg2":
+            print(json.dumps(extras))
+            return
+
+    if (not args.no_extras and args.only == "") or args.only == "grouped":
 
         wl4 = W.cfg4()
         xq4, xs4 = mslk_amd.quantize_fp8_row(wl4.x.to(dev), use_triton=False)
@@ -449,12 +546,16 @@ def main():
         xl, sl = list(xq4.split(wl4.counts)), list(xs4.split(wl4.counts))
         ys4 = torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4)
         call4 = api.grouped_call(xl, wq4, sl, ws4, ys4)
-        for _ in range(40):   # the first few dozen launches on freshly allocated 640 MiB of weights run up to 25 % slower
-            call4()
+        _settle(lambda i: call4())   # the first few dozen launches on freshly allocated 640 MiB of weights run up to 25 % slower
         ms = _median_events_ms(lambda i: call4(), 10)
         f4 = 2.0 * 8192 * 8192 * 5120
+        par4 = [_parity(ys4[e], xl[e], wq4[e], sl[e], ws4[e]) for e in range(16) if wl4.counts[e]]
         extras["grouped_cfg4_16x8192x5120"] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12,
-                                                "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS, "counts": wl4.counts}
+                                                "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS, "counts": wl4.counts,
+                                                "parity": {"max_rel": max(p["max_rel"] for p in par4),
+                                                           "normwise": max(p["normwise"] for p in par4),
+                                                           "elementwise_violations": sum(p["elementwise_violations"] for p in par4),
+                                                           "elements": sum(p["elements"] for p in par4)}}
         # the same experts through the device-resident group layouts (no host knowledge of the sizes),
         # and as a uniform batch of 16 x [512 x 8192 x 5120] (same FLOPs, no ragged tiles)
         WQ4, WS4 = torch.stack(wq4), torch.stack(ws4)
@@ -478,11 +579,13 @@ def main():
 
         for name, call in (("grouped_stacked_cfg4", stacked_call), ("grouped_mm_2d3d_cfg4", offsets_call),
                            ("batched_16x512x8192x5120", batched_call)):
-            for _ in range(40):
-                call()
+            _settle(lambda i: call(), 20.0)
             ms = _median_events_ms(lambda i: call(), 10)
             extras[name] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12, "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS}
         del WQ4, wl4
+        if args.only == "grouped":
+            print(json.dumps(extras))
+            return
 
     # ---------------------------------------------------------------- CPU baseline
     cpu = None
@@ -496,7 +599,9 @@ def main():
         "dtype": "fp8_e4m3fn x fp8_e4m3fn -> fp32 accumulate -> bf16", "data": "synthetic",
         "config": {"workload": "cfg1: f8f8bf16_rowwise M=N=K=4096, x ~ N(0,1) with 1% K-channels x20 quantized by "
                                "quantize_fp8_row, w ~ N(0,0.02) pre-quantized; one step = one GEMM call via the C ABI, "
-                               f"rotating over {NSETS} operand sets ({NSETS * 64} MiB); quantize timed separately (see extras)"},
+                               f"rotating over {NSETS} operand sets ({NSETS * 64} MiB); quantize timed separately (see extras); "
+                               f"before the --warmup steps an untimed clock-settling phase of the same launches runs until "
+                               f"{SETTLE_MS:.0f} ms of GPU time have passed ({settle_launches} launches in this run)"},
         "pct_of_fp8_peak_5.0PF": 100.0 * value * 1e12 / PEAK_FP8_FLOPS,
         "pct_of_reference_peak_4.6PF": 100.0 * value * 1e12 / PEAK_FP8_FLOPS_REF,
         "roofline": {"kernel": "dense_tiled_kernel<256,256> (f8f8bf16_rowwise 4096^3)", "bound": "mfma",

@@ -162,6 +162,23 @@ int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, con
 size_t mslk_amd_static_scratch_bytes(void);
 
 /*
+ * Decode fast path: row-wise quantization of the activations AND the GEMM in one launch.  Replaces the pair
+ * quantize_fp8_row(x) -> f8f8bf16_rowwise(xq, wq, x_scale, w_scale) that callers of the reference issue for every
+ * decode step (reference: bench/gemm/gemm_ops.py:593-673; mslk/moe/layers.py:1096,1123), for the shapes where the first
+ * launch costs about as much as the work: 1 <= M <= 4, K % 1024 == 0 (mslk_amd_quantize_f8f8bf16_rowwise_supported).
+ *   x    [M, K] bf16 (x_dtype must be MSLK_AMD_DTYPE_BF16), row stride x_row_stride elements (a multiple of 8), 16-byte aligned
+ *   wq, w_scale, bias, y   as mslk_amd_f8f8bf16_rowwise
+ *   xq_out [M, K] e4m3fn, x_scale_out [M] fp32: optional (NULL to skip); they receive the codes and scales the kernel
+ *          multiplied with -- the bits mslk_amd_quantize_fp8_row produces for x (no scale_ub).
+ * Every workgroup quantizes the M rows itself (they stay in L2; each wave converts the K steps it multiplies), so nothing is exchanged between workgroups and the
+ * call is one kernel: no workspace, graph-safe.  Other shapes return an error; use the two entry points then.
+ */
+int mslk_amd_quantize_f8f8bf16_rowwise(const void* x, int x_dtype, int64_t x_row_stride, const void* wq, const float* w_scale,
+                                       const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                                       void* xq_out, float* x_scale_out, void* stream);
+int mslk_amd_quantize_f8f8bf16_rowwise_supported(int64_t M, int64_t N, int64_t K);
+
+/*
  * The same GEMM with an fp16 (IEEE half, round to nearest even, overflow to infinity) output.
  * Replaces mslk::gemm::f8f8f16_rowwise (reference: csrc/gemm/gemm_ops.cpp:88-89,
  * csrc/gemm/ck/fp8_rowwise/fp8fp8fp16_rowwise_gemm.hip:66-133).  Arguments as above (the same workspace rule); y is fp16.

@@ -35,6 +35,9 @@ SIGNATURES = {
     "mslk_amd_f8f8bf16_rowwise_static_scratch": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                                          c_int64, c_int64, c_int64, c_void_p]),
     "mslk_amd_static_scratch_bytes": (c_size_t, []),
+    "mslk_amd_quantize_f8f8bf16_rowwise": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                                   c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p]),
+    "mslk_amd_quantize_f8f8bf16_rowwise_supported": (c_int, [c_int64, c_int64, c_int64]),
     "mslk_amd_f8f8f16_rowwise": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
                                          c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "mslk_amd_f8f8_rowwise_preshuffle": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,

@@ -248,6 +248,27 @@ int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, con
   return rowwise_impl(op, 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, ptr, bytes, stream);
 }
 
+int mslk_amd_quantize_f8f8bf16_rowwise_supported(int64_t M, int64_t N, int64_t K) {
+  return M >= 1 && M <= 4 && N >= 1 && N <= kIntMax && K >= 1024 && K % 1024 == 0 && K <= (int64_t(1) << 25);
+}
+
+int mslk_amd_quantize_f8f8bf16_rowwise(const void* x, int x_dtype, int64_t x_row_stride, const void* wq, const float* w_scale,
+                                       const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
+                                       void* xq_out, float* x_scale_out, void* stream) {
+  const char* op = "quantize_f8f8bf16_rowwise";
+  if (x_dtype != MSLK_AMD_DTYPE_BF16) return fail("%s: activations must be bf16 (dtype code %d)", op, x_dtype);
+  if (bias_dtype < 0 || bias_dtype > 2) return fail("%s: bad bias dtype code %d", op, bias_dtype);
+  if ((bias_dtype != 0) != (bias != nullptr)) return fail("%s: bias pointer and bias dtype disagree", op);
+  if (!mslk_amd_quantize_f8f8bf16_rowwise_supported(M, N, K))
+    return fail("%s: the one-launch path needs 1 <= M <= 4 and K a multiple of 1024 (got M=%lld, N=%lld, K=%lld); "
+                "use mslk_amd_quantize_fp8_row followed by mslk_amd_f8f8bf16_rowwise", op, (long long)M, (long long)N, (long long)K);
+  if (!x || !wq || !w_scale || !y) return fail("%s: null pointer", op);
+  GemmProblem p{nullptr, (const uint8_t*)wq, nullptr, w_scale, bias, (uint16_t*)y, (int)M, (int)N, (int)K, bias_dtype, 0, 0};
+  if (!skinny_fused_quant_supports(p, x, x_row_stride) || (xq_out && reinterpret_cast<uintptr_t>(xq_out) % 16 != 0))
+    return fail("%s: x, wq and xq_out must be 16-byte aligned and the row stride of x a multiple of 8 elements, at least K", op);
+  return check_hip(launch_skinny_fused_quant(p, x, x_row_stride, xq_out, x_scale_out, (hipStream_t)stream), "fused decode launch");
+}
+
 int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                              const void* bias, int bias_dtype, void* y, int64_t M, int64_t N, int64_t K,
                              void* workspace, size_t workspace_bytes, void* stream) {

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
   int tm, tn;
   local_tile(t - d.tile_begin, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  GemmTile<TS, 0> tile;
+  GemmTile<TS, 0, false, true> tile;   // ROWSKIP: the ragged last row tile of a group costs what its rows cost
   tile.run(lds, d.xq + (int64_t)m0 * d.K, d.wq + (int64_t)n0 * d.K, d.xs + m0, d.ws + n0, nullptr,
            d.y + (int64_t)m0 * d.N + n0, d.M - m0, d.N - n0, d.N, d.K);
 }
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(256) void grouped_device_kernel(DeviceGroups p) {
     slow_tile<BM, BN, BIAS>(a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, K);
     return;
   }
-  GemmTile<TS, BIAS> tile;
+  GemmTile<TS, BIAS, false, true> tile;
   tile.run(lds, a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, (uint32_t)p.K);
 }
 

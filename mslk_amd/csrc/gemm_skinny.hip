@@ -18,6 +18,7 @@
 //   * the eight per-wave partial sums meet in LDS; the lanes reduce, scale and store bf16.
 #include "common.h"
 #include "kernels.h"
+#include "quant_math.h"
 
 namespace mslk_amd {
 namespace {
@@ -374,7 +375,222 @@ hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
   return hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------------------------
+// Decode with the activation quantizer fused in: bf16 activations in, M <= 4, K % 1024 == 0.
+//
+// The reference quantizes the activations with one launch and multiplies with a second
+// (bench/gemm/gemm_ops.py:593-673); at decode sizes the first launch costs about a third of the pair.  Here every
+// workgroup quantizes the (at most 4) activation rows itself, with the arithmetic of the stand-alone quantizer
+// (mslk/quantize/triton/fp8_quantize.py:356-378; the codes and scales are the same bits):
+//   1. row maxima: the 512 lanes sweep each row with 16-byte loads (the rows stay in L2: M * K * 2 bytes in all),
+//      wave reduction, partial maxima meet in LDS, every lane picks up the multipliers of the M rows;
+//   2. the weight stream as in skinny_lds_kernel (DMA into wave-private LDS).  A wave owns the K steps
+//      wave, wave + 8, ...: next to their weight loads it fetches the bf16 activations of just these steps (M * 256 bytes
+//      per step, 8 elements per lane and load), converts them in registers and parks the codes in its private LDS
+//      buffer, from where the MFMA fragment is two 16-byte reads.  The conversion work of a workgroup is therefore M * K
+//      elements split over its 512 lanes.  No scale_ub here, so no product exceeds 448 (1 + 2^-22) and the conversion
+//      needs no overflow fix-up; NaN stays NaN.
+// Workgroup 0 also writes the codes and the scales out when the caller wants them.
+// ---------------------------------------------------------------------------------------------
+MSLK_AMD_DEVINL v2i quantize8_bf16(v4i raw, float inv) {
+  const uint32_t w[4] = {(uint32_t)raw.x, (uint32_t)raw.y, (uint32_t)raw.z, (uint32_t)raw.w};
+  float f[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    f[2 * j] = __uint_as_float(w[j] << 16) * inv;
+    f[2 * j + 1] = __uint_as_float(w[j] & 0xFFFF0000u) * inv;
+  }
+  int lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false);
+  lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+  int hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
+  hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+  return v2i{lo, hi};
+}
+
+constexpr int kFusedMaxM = 4;
+
+template <int U, int BIAS>
+__global__ __launch_bounds__(512) void skinny_fused_quant_kernel(GemmProblem p, const uint16_t* __restrict__ x, int64_t x_stride,
+                                                                 uint8_t* __restrict__ xq_out, float* __restrict__ xs_out) {
+  constexpr int kWaves = 8;
+  constexpr int WBYTES = U * 2048;                       // U weight tiles (16 rows x 128 B) of one K step each
+  constexpr int CBYTES = U * kFusedMaxM * 128;           // codes of up to 4 activation rows for the same U steps
+  constexpr int XBUF = WBYTES + CBYTES;                  // 10 KiB per wave at U = 4: two workgroups fill the LDS of a CU exactly
+  constexpr int NCH = U * kFusedMaxM * 16 / 64;          // 16-byte bf16 chunks (8 elements) per lane and batch, at most
+  __shared__ __attribute__((aligned(1024))) char lds[kWaves * XBUF];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int i = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16;
+  const int K = p.K, M = p.M;
+  char* xbuf = lds + wave * XBUF;
+  // small arrays of the set-up phase live in the staging area, which the weight stream only starts to fill after the
+  // last barrier of the set-up
+  uint32_t* amax_part = reinterpret_cast<uint32_t*>(lds);              // [4][8]
+  float* row_inv = reinterpret_cast<float*>(lds + 256);                // [4]
+  float* row_scale = reinterpret_cast<float*>(lds + 256 + 16);         // [4]
+
+  // weight rows of this workgroup as DMA source offsets (see skinny_lds_kernel)
+  uint32_t w_off[2];
+  const uint8_t* w_base = p.wq + (int64_t)n0 * K;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int r = 8 * h + (lane >> 3);
+    w_off[h] = (uint32_t)(n0 + r < p.N ? r : p.N - 1 - n0) * (uint32_t)K + (((lane & 7) ^ row_swz(r)) << 4);
+  }
+  const int xr0 = i * 128 + ((g ^ row_swz(i)) << 4);
+  const int xr1 = i * 128 + (((g + 4) ^ row_swz(i)) << 4);
+
+  // epilogue operands first: their latency hides behind the quantizer
+  const int t = threadIdx.x & 255;
+  const int e_n = n0 + 4 * (t >> 6) + (t & 3);
+  const int e_m = (t >> 2) & 15;
+  const bool e_ok = threadIdx.x < 256 && e_n < p.N && e_m < M;
+  const float e_ws = e_ok ? p.ws[e_n] : 0.f;
+  float e_b = 0.f;
+  if constexpr (BIAS == 1) e_b = e_ok ? reinterpret_cast<const float*>(p.bias)[e_n] : 0.f;
+  if constexpr (BIAS == 2) e_b = e_ok ? bf16_bits_to_f32(reinterpret_cast<const uint16_t*>(p.bias)[e_n]) : 0.f;
+
+  // 1. row maxima (as raw bf16 bits: unsigned order equals numeric order for non-negative values, NaN sorts last)
+  const int chunks = K >> 3;
+  for (int r = 0; r < M; ++r) {
+    const v4i* xr = reinterpret_cast<const v4i*>(x + (int64_t)r * x_stride);
+    us2 acc2 = {0, 0};
+    for (int c = threadIdx.x; c < chunks; c += kWaves * 64) {
+      const v4i v = xr[c];
+      const uint32_t w4[4] = {(uint32_t)v.x, (uint32_t)v.y, (uint32_t)v.z, (uint32_t)v.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc2 = __builtin_elementwise_max(acc2, __builtin_bit_cast(us2, w4[j] & 0x7FFF7FFFu));
+    }
+    uint32_t m = __builtin_bit_cast(uint32_t, acc2);
+    m = max(m & 0xFFFFu, m >> 16);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) m = max(m, (uint32_t)__shfl_xor((int)m, off, 64));
+    if (lane == 0) amax_part[r * kWaves + wave] = m;
+  }
+  __syncthreads();
+  if (threadIdx.x < M) {
+    uint32_t mb = amax_part[threadIdx.x * kWaves];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) mb = max(mb, amax_part[threadIdx.x * kWaves + w]);
+    float inv, sc;
+    scales_from_amax<0, false>(bf16_bits_to_f32(mb), nullptr, 0.f, inv, sc);
+    row_inv[threadIdx.x] = inv;
+    row_scale[threadIdx.x] = sc;
+    if (blockIdx.x == 0 && xs_out != nullptr) xs_out[threadIdx.x] = sc;
+  }
+  __syncthreads();
+  float inv_r[kFusedMaxM];
+#pragma unroll
+  for (int r = 0; r < kFusedMaxM; ++r) inv_r[r] = row_inv[r < M ? r : 0];
+  const float e_xs = row_scale[e_m < M ? e_m : 0];
+  __syncthreads();   // the staging area is free for the weight stream from here on
+
+  // This lane's chunks of a batch: chunk c = (step u of the batch, row, 8-element column block) -- the same for every batch.
+  const bool write_codes = blockIdx.x == 0 && xq_out != nullptr;
+  const int per_step = M * 16;                         // chunks per K step
+  int64_t c_src[NCH];                                  // element offset into x, less the K offset of the batch
+  int c_dst[NCH];                                      // byte offset into the wave's code area; -1: no chunk
+  int64_t c_out[NCH];                                  // byte offset into xq_out, less the K offset of the batch
+  float c_inv[NCH];
+#pragma unroll
+  for (int j = 0; j < NCH; ++j) {
+    const int c = lane + j * 64;
+    const int u = c / per_step, rem = c - u * per_step;
+    const int row = rem >> 4, col = rem & 15;
+    const bool ok = u < U;
+    c_src[j] = (int64_t)row * x_stride + u * kWaves * kStep + col * 8;
+    c_out[j] = (int64_t)row * K + u * kWaves * kStep + col * 8;
+    c_dst[j] = ok ? (u * kFusedMaxM + row) * 128 + col * 8 : -1;
+    c_inv[j] = row == 0 ? inv_r[0] : row == 1 ? inv_r[1] : row == 2 ? inv_r[2] : inv_r[3];
+  }
+  char* cbuf = xbuf + WBYTES;
+  const char* xfrag = cbuf + (i < M ? i : M - 1) * 128 + g * 16;   // fragment rows beyond M repeat the last row; never stored
+
+  // 2. weight stream; K % (8 * 128) == 0: every wave owns KT / 8 complete steps
+  v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
+  const int KT = K / kStep;
+  for (int kt0 = wave; kt0 < KT; kt0 += kWaves * U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = kt0 + u * kWaves;
+      if (kt < KT) {           // wave-uniform
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+          __builtin_amdgcn_global_load_lds((gbl_ptr_t)(w_base + kt * kStep + w_off[h]), (lds_ptr_t)(xbuf + (u * 2 + h) * 1024), 16, 0, 0);
+      }
+    }
+    const int steps_left = (KT - kt0 + kWaves - 1) / kWaves;       // K steps of this batch that exist (wave-uniform), >= 1
+    v4i raw[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const bool ok = c_dst[j] >= 0 && (c_dst[j] >> 9) < steps_left;   // 512 bytes of codes per step
+      raw[j] = v4i{0, 0, 0, 0};
+      if (ok) raw[j] = *reinterpret_cast<const v4i*>(x + c_src[j] + (int64_t)kt0 * kStep);
+    }
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's loads have landed
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+      const bool ok = c_dst[j] >= 0 && (c_dst[j] >> 9) < steps_left;
+      if (ok) {
+        const v2i q = quantize8_bf16(raw[j], c_inv[j]);
+        *reinterpret_cast<v2i*>(cbuf + c_dst[j]) = q;
+        if (write_codes) *reinterpret_cast<v2i*>(xq_out + c_out[j] + (int64_t)kt0 * kStep) = q;
+      }
+    }
+    // the codes were written by other lanes of this wave: LDS operations of a wave complete in order, no barrier needed
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int kt = kt0 + u * kWaves;
+      if (kt < KT) {
+        const char* wt = xbuf + u * 2048;
+        const v4i wlo = *reinterpret_cast<const v4i*>(wt + xr0);
+        const v4i whi = *reinterpret_cast<const v4i*>(wt + xr1);
+        const v4i xlo = *reinterpret_cast<const v4i*>(xfrag + u * kFusedMaxM * 128);
+        const v4i xhi = *reinterpret_cast<const v4i*>(xfrag + u * kFusedMaxM * 128 + 64);
+        const v8i wf = __builtin_shufflevector(wlo, whi, 0, 1, 2, 3, 4, 5, 6, 7);
+        const v8i xf = __builtin_shufflevector(xlo, xhi, 0, 1, 2, 3, 4, 5, 6, 7);
+        acc = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf, acc, 0, 0, 0, 0, 0, 0);
+      }
+    }
+  }
+
+  // reduction across the 8 waves in their (now dead) staging buffers, then scale, bias and store
+  *reinterpret_cast<v4f*>(reinterpret_cast<float*>(xbuf) + lane * 4) = acc;
+  __syncthreads();
+  if (e_ok) {
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) sum += reinterpret_cast<const float*>(lds + w * XBUF)[t];
+    float val = (sum * e_ws) * e_xs;
+    if constexpr (BIAS != 0) val += e_b;
+    p.y[(int64_t)e_m * p.N + e_n] = (uint16_t)f32_to_out_bits(val, p.out_f16);
+  }
+}
+
 }  // namespace
+
+bool skinny_fused_quant_supports(const GemmProblem& p, const void* x, int64_t x_stride) {
+  return p.M >= 1 && p.M <= kFusedMaxM && p.N >= 1 && p.K >= 1024 && p.K % (8 * kStep) == 0 &&
+         (int64_t)64 * p.K < (int64_t(1) << 32) && !p.w_preshuffled && x_stride >= p.K && x_stride % 8 == 0 &&
+         reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0;
+}
+
+hipError_t launch_skinny_fused_quant(const GemmProblem& p, const void* x, int64_t x_stride, void* xq_out, float* xs_out,
+                                     hipStream_t s) {
+  if (!skinny_fused_quant_supports(p, x, x_stride)) return hipErrorInvalidValue;
+  if (xq_out != nullptr && reinterpret_cast<uintptr_t>(xq_out) % 8 != 0) return hipErrorInvalidValue;
+  constexpr int U = 4;
+  const uint16_t* xb = static_cast<const uint16_t*>(x);
+  uint8_t* q = static_cast<uint8_t*>(xq_out);
+  const unsigned grid = (unsigned)((p.N + 15) / 16);
+  switch (p.bias_dtype) {
+    case 0: skinny_fused_quant_kernel<U, 0><<<grid, 512, 0, s>>>(p, xb, x_stride, q, xs_out); break;
+    case 1: skinny_fused_quant_kernel<U, 1><<<grid, 512, 0, s>>>(p, xb, x_stride, q, xs_out); break;
+    default: skinny_fused_quant_kernel<U, 2><<<grid, 512, 0, s>>>(p, xb, x_stride, q, xs_out); break;
+  }
+  return hipGetLastError();
+}
 
 bool skinny_supports(const GemmProblem& p) {
   if (p.w_preshuffled && (p.N % 16 != 0 || p.K % 64 != 0)) return false;

@@ -19,9 +19,10 @@
 //     WQ tiles of steps k+1 and k+2 are in flight (the weights are the cold, read-once stream).
 // Rows
 //   * The 16-row m fragments of a tile are dealt to the wave rows round-robin (wave row wm owns fragments wm, wm + WM,
-//     ...), and a tile with fewer valid rows than BM skips the MFMAs, the fragment reads, the DMA loads and the epilogue
-//     work of fragments that hold no valid row: the cost of a ragged tile (the last row tile of an MoE group) follows its
-//     row count in steps of 16 * WM rows, down to what the weight stream alone costs.
+//     ...).  With ROWSKIP a tile with fewer valid rows than BM runs a K loop compiled for a quarter, half or three
+//     quarters of the m fragments per wave and leaves out the XQ loads and the epilogue work of fragments without valid
+//     rows: the cost of a ragged tile (the last row tile of an MoE group) follows its row count in steps of BM / 4 rows,
+//     down to what the weight stream alone costs.
 // Math
 //   * v_mfma_f32_16x16x128_f8f6f4 (both operands e4m3, unit block scales).  WQ rows are the first
 //     operand and XQ rows the second, so a lane ends up holding 4 consecutive n for one m.
@@ -88,14 +89,13 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
 // MFMA operand read it (reference: mslk/quantize/shuffle.py:182-246).  One DMA then moves one block
 // (1 KiB contiguous in HBM and in LDS), the WQ fragment read is lane-linear, and both operands give
 // lane (i, g) the k bytes [16 g, 16 g + 16) and [64 + 16 g, 64 + 16 g + 16) of row i.
-template <typename TS, int BIAS, bool PS = false>
+template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false>
 struct GemmTile {
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
   uint32_t b_off[TS::LB];
   int out_f16 = 0;          // output element type: 0 bf16, 1 fp16 (set by the caller before run())
-  int a_rows = TS::kBM;     // valid rows of the XQ tile (wave-uniform); DMA loads of 8-row groups beyond them are skipped
-  int fmv = TS::FM;         // m fragments of this wave that hold at least one valid row (wave-uniform)
+  int a_rows = TS::kBM;     // valid rows of the XQ tile (wave-uniform)
   const uint8_t* a_base;    // XQ + m0 * K   (wave-uniform)
   const uint8_t* b_base;    // WQ + n0 * K
 
@@ -108,11 +108,6 @@ struct GemmTile {
     a_base = xq_tile;
     b_base = wq_tile;
     a_rows = rows_a;
-    {
-      const int nf = (rows_a + 15) >> 4;                      // fragments of the tile with a valid row
-      const int mine = (nf - wave / TS::WN + TS::WM - 1) / TS::WM;   // of which this wave row owns fragments wm, wm + WM, ...
-      fmv = mine < 0 ? 0 : (mine > TS::FM ? TS::FM : mine);
-    }
 #pragma unroll
     for (int i = 0; i < TS::LA; ++i) {
       const int row = (wave * TS::LA + i) * 8 + (lane >> 3);
@@ -142,20 +137,21 @@ struct GemmTile {
 
   // DMA load number i (0 .. LA-1 for the XQ tile, 0 .. LB-1 for the WQ tile) of the K step at byte k0.
   // `abuf` / `bbuf` are the LDS buffers that receive the XQ / WQ tile of the K step at byte k0.
-  // RAGGED: the 8 rows of a load that lie beyond the valid rows of the tile are not fetched (nobody multiplies them).
-  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void issue_a(char* abuf, int k0, int i) {
-    if (RAGGED && (wave_id() * TS::LA + i) * 8 >= a_rows) return;   // wave-uniform
     dma16(a_base + k0 + a_off[i], abuf + (wave_id() * TS::LA + i) * 1024);
   }
   MSLK_AMD_DEVINL void issue_b(char* bbuf, int k0, int i) {
     // pre-shuffled: the K step at byte k0 starts 16 rows x k0 bytes into the row group
     dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
   }
-  template <bool RAGGED = false>
   MSLK_AMD_DEVINL void issue_a_all(char* abuf, int k0) {
 #pragma unroll
-    for (int i = 0; i < TS::LA; ++i) issue_a<RAGGED>(abuf, k0, i);
+    for (int i = 0; i < TS::LA; ++i) issue_a(abuf, k0, i);
+  }
+  // Ragged tiles: a wave whose share of the XQ tile (8 * LA consecutive rows) starts beyond the valid rows fetches
+  // nothing -- nobody multiplies those rows (one wave-uniform branch for the wave's loads of a step).
+  MSLK_AMD_DEVINL void issue_a_live(char* abuf, int k0) {
+    if (wave_id() * TS::LA * 8 < a_rows) issue_a_all(abuf, k0);
   }
   MSLK_AMD_DEVINL void issue_b_all(char* bbuf, int k0) {
 #pragma unroll
@@ -224,13 +220,12 @@ struct GemmTile {
     return bbuf + (wave_id() % TS::WN) * (TS::kBN / TS::WN) * kBK;
   }
   // First fragments of a K step: all XQ fragments and WQ fragment 0.
-  template <bool RAGGED = false>
+  template <int FMV = TS::FM>
   MSLK_AMD_DEVINL void load_first_frags(const char* abuf, const char* bbuf, v8i (&xf)[TS::FM], v8i& wf0) {
     const FragOff fo = frag_off();
     wf0 = load_frag_b(b_tile_of(bbuf), 0, fo);
 #pragma unroll
-    for (int tm = 0; tm < TS::FM; ++tm)
-      if (!RAGGED || tm < fmv) xf[tm] = load_frag_a(a_tile_of(abuf), tm, fo);
+    for (int tm = 0; tm < FMV; ++tm) xf[tm] = load_frag_a(a_tile_of(abuf), tm, fo);
   }
 
   // Waits until at most `pending` of this wave's DMA loads (the youngest ones) are still in flight and
@@ -263,11 +258,14 @@ struct GemmTile {
   //     fragments already on their way.
   // In the symmetric ring (TileShape::RING) the XQ loads go to `a_dst` != `a_nxt` as well, and PENDING, the
   // number of this wave's youngest loads that may still be in flight at the barrier, covers RING - 2 steps.
-  // RAGGED: the tile has fewer than BM valid rows; MFMAs and XQ fragment reads of this wave's fragments >= fmv are
-  // skipped (wave-uniform branches) and so are the DMA loads of XQ rows nobody multiplies.
-  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING, bool RAGGED = false>
+  // FMV < FM: a ragged tile, only the first FMV m fragments of every wave hold valid rows -- see step_rows().
+  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING, int FMV = TS::FM>
   MSLK_AMD_DEVINL void step(const char* b_cur, char* a_dst, const char* a_nxt, const char* b_nxt, char* b_far, int k_a,
                             int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
+    if constexpr (FMV < TS::FM) {
+      step_rows<DMA_A, DMA_B, NEXT, PENDING, FMV>(b_cur, a_dst, a_nxt, b_nxt, b_far, k_a, k_b, acc, xf, wf0);
+      return;
+    }
     constexpr int HALF = TS::FN / 2;
     static_assert((TS::LA + TS::LB) % HALF == 0, "DMA loads spread evenly over the first half");
     constexpr int NDMA = (TS::LA + TS::LB) / HALF;   // DMA loads per MFMA group
@@ -286,8 +284,7 @@ struct GemmTile {
       v8i wf_next;
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) {
-        if (!RAGGED || tm < fmv)
-          acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+        acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
         if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
         const int d = tm - (TS::FM - SLOTS);
         if (tn < HALF && d >= 0) {
@@ -296,7 +293,7 @@ struct GemmTile {
             const int q = tn * NDMA + d * PER_SLOT + j;   // all XQ loads are older than all WQ loads of the step
             if (d * PER_SLOT + j < NDMA) {
               if (q < TS::LA) {
-                if constexpr (DMA_A) issue_a<RAGGED>(a_dst, k_a, q);
+                if constexpr (DMA_A) issue_a(a_dst, k_a, q);
               } else {
                 if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
               }
@@ -315,11 +312,53 @@ struct GemmTile {
     const char* a_next = a_tile_of(a_nxt);
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
-      if (!RAGGED || tm < fmv) {
-        acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
-        if constexpr (NEXT) xf[tm] = load_frag_a(a_next, tm, fo);
+      acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+      if constexpr (NEXT) {
+        xf[tm] = load_frag_a(a_next, tm, fo);
+        __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
       }
-      if constexpr (NEXT) __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
+  // One K step of a ragged tile: as step(), but every n fragment multiplies only the first FMV m fragments of the wave,
+  // the XQ loads of the next step follow the first MFMA group as one block (left out by waves whose rows are all
+  // beyond the valid ones) and the WQ loads follow the second.  Such a step is short: it waits for memory rather than
+  // for the matrix cores, so the fine interleave of step() would buy nothing.
+  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING, int FMV>
+  MSLK_AMD_DEVINL void step_rows(const char* b_cur, char* a_dst, const char* a_nxt, const char* b_nxt, char* b_far, int k_a,
+                                 int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
+    static_assert(TS::FN >= 3 && FMV >= 1 && FMV < TS::FM, "ragged step");
+    const FragOff fo = frag_off();
+    const char* b_tile = b_tile_of(b_cur);
+    v8i wf = wf0;
+#pragma unroll
+    for (int tn = 0; tn < TS::FN - 1; ++tn) {
+      const v8i wf_next = load_frag_b(b_tile, tn + 1, fo);
+#pragma unroll
+      for (int tm = 0; tm < FMV; ++tm)
+        acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
+      if (tn == 0) {
+        if constexpr (DMA_A) issue_a_live(a_dst, k_a);   // all XQ loads are older than all WQ loads of the step
+      }
+      if (tn == 1) {
+        if constexpr (DMA_B) issue_b_all(b_far, k_b);
+      }
+      wf = wf_next;
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if constexpr (NEXT) {
+      wait_and_barrier<PENDING>();
+      wf0 = load_frag_b(b_tile_of(b_nxt), 0, fo);
+    }
+    const char* a_next = a_tile_of(a_nxt);
+#pragma unroll
+    for (int tm = 0; tm < FMV; ++tm) {
+      acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+      if constexpr (NEXT) {
+        xf[tm] = load_frag_a(a_next, tm, fo);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
@@ -336,40 +375,51 @@ struct GemmTile {
                            const float* ws, const void* bias, uint16_t* y, int m_rem, int n_rem, int N, int K,
                            uint32_t ld) {
     v4f acc[TS::FN][TS::FM];
-    // A tile with fewer valid rows than BM takes the K loop that skips the fragments without valid rows.
-    if constexpr (TS::RING == 0) {
-      if (m_rem < TS::kBM) accumulate<true>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
-      else accumulate<false>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
-    } else {
-      accumulate<false>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
-    }
+    accumulate_rows(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
+  }
+
+  // K loop of a tile with m_rem valid rows.
+  MSLK_AMD_DEVINL void accumulate_rows(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
+                                       uint32_t ld, v4f (&acc)[TS::FN][TS::FM]) {
+    // A tile with at most three quarters of its rows takes a K loop compiled for fewer m fragments per wave: the
+    // fragments are dealt to the wave rows round-robin, so m_rem rows need ceil(ceil(m_rem / 16) / WM) of them.
+    if constexpr (ROWSKIP && TS::RING == 0 && TS::FM % 4 == 0) {
+      constexpr int Q = TS::kBM / 4;
+      if (m_rem > 3 * Q) accumulate<TS::FM>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+      else if (m_rem > 2 * Q) accumulate<3 * TS::FM / 4>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+      else if (m_rem > Q) accumulate<TS::FM / 2>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+      else accumulate<TS::FM / 4>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    } else {
+      accumulate<TS::FM>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    }
   }
 
   // K loop only: acc = sum over the K bytes of the operand rows starting at xq_tile / wq_tile.  Ends with a
   // workgroup barrier, after which the LDS buffers are dead.
-  template <bool RAGGED = false>
+  template <int FMV = TS::FM>
   MSLK_AMD_DEVINL void accumulate(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
                                   uint32_t ld, v4f (&acc)[TS::FN][TS::FM]) {
     if constexpr (TS::RING == 0) {
-      prologue<RAGGED>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld);
+      prologue<(FMV < TS::FM)>(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld);
     } else {
       init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
     }
-    accumulate_issued<false, RAGGED>(lds, K, acc);
+    accumulate_issued<false, FMV>(lds, K, acc);
   }
 
   // Two-plus-three buffers only: per-lane addresses of a tile and the first DMA loads of its K loop (step 0 of both
   // operands, step 1 of WQ) into the buffers the loop starts from.  A persistent workgroup calls this for its next
   // tile before the epilogue of the current one, which must then stay out of those three buffers.
-  template <bool RAGGED = false>
+  template <bool LIVE_ROWS_ONLY = false>
   MSLK_AMD_DEVINL void prologue(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
                                 uint32_t ld) {
     static_assert(TS::RING == 0, "the symmetric ring issues its own prologue");
     init(xq_tile, wq_tile, m_rem < TS::kBM ? m_rem : TS::kBM, n_rem < TS::kBN ? n_rem : TS::kBN, ld);
     const int KT = K / kBK;
     if (KT > 0) {
-      issue_a_all<RAGGED>(lds, 0);
+      if constexpr (LIVE_ROWS_ONLY) issue_a_live(lds, 0);
+      else issue_a_all(lds, 0);
       issue_b_all(lds + 2 * TS::A_BYTES, 0);
       if (KT > 1) issue_b_all(lds + 2 * TS::A_BYTES + TS::B_BYTES, kBK);
     }
@@ -378,9 +428,9 @@ struct GemmTile {
   // K loop after prologue() (or, for the symmetric ring, after init()).  DRAIN: the wave has other memory
   // operations in flight behind the prologue loads (the stores of the previous tile's epilogue), so the first wait
   // is for all of them instead of "all but the youngest WQ loads".
-  template <bool DRAIN, bool RAGGED = false>
+  template <bool DRAIN, int FMV = TS::FM>
   MSLK_AMD_DEVINL void accumulate_issued(char* lds, int K, v4f (&acc)[TS::FN][TS::FM]) {
-    static_assert(!RAGGED || TS::RING == 0, "row skipping is built for the two-plus-three buffer tiles");
+    static_assert(FMV == TS::FM || TS::RING == 0, "row skipping is built for the two-plus-three buffer tiles");
 #pragma unroll
     for (int tn = 0; tn < TS::FN; ++tn)
 #pragma unroll
@@ -400,19 +450,19 @@ struct GemmTile {
       if (KT > 0) {
         if (KT > 1 && !DRAIN) wait_and_barrier<TS::LB>();
         else wait_and_barrier<0>();
-        load_first_frags<RAGGED>(a_cur, b_cur, xf, wf0);
+        load_first_frags<FMV>(a_cur, b_cur, xf, wf0);
         // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
         for (int kt = 0; kt < KT - 2; ++kt) {
-          step<true, true, true, TS::LB, RAGGED>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
+          step<true, true, true, TS::LB, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
         if (KT > 1) {
-          step<true, false, true, 0, RAGGED>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
+          step<true, false, true, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
-        step<false, false, false, 0, RAGGED>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
+        step<false, false, false, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
       }
     } else {
       // Symmetric ring: buffer i % RING holds step i; step kt fetches step kt + RING - 1 into the buffers step
@@ -454,8 +504,8 @@ struct GemmTile {
       __syncthreads();   // everybody is done with the buffers of the full steps before one pair is refilled
       issue_loads_tail(a_tail, b_tail, KT * kBK, k_tail);
       __syncthreads();
-      load_first_frags<RAGGED>(a_tail, b_tail, xf, wf0);
-      step<false, false, false, 0, RAGGED>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
+      load_first_frags<FMV>(a_tail, b_tail, xf, wf0);
+      step<false, false, false, 0, FMV>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
     }
     __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
   }

@@ -65,6 +65,11 @@ bool skinny_supports(const GemmProblem& p);
 // (measured crossover: streaming wins at N = 4096, tiles from N = 5120 on).
 constexpr int kShortTileMinN = 5120;
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s);
+// Decode with the activation quantizer fused in: `x` holds p.M <= 4 rows of p.K bf16 (row stride x_stride elements);
+// p.xq / p.xs are not read.  xq_out [M, K] / xs_out [M] (optional) receive the codes and scales the kernel multiplied with.
+bool skinny_fused_quant_supports(const GemmProblem& p, const void* x, int64_t x_stride);
+hipError_t launch_skinny_fused_quant(const GemmProblem& p, const void* x, int64_t x_stride, void* xq_out, float* xs_out,
+                                     hipStream_t s);
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s);   // any shape, slow
 hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s);
 // dst[r, 0:K] = src[r, 0:K], dst[r, K:Kp] = 0 for `rows` rows of bytes (Kp a multiple of 16, dst 16-byte aligned)

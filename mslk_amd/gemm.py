@@ -35,6 +35,8 @@ _SCHEMAS = {
     "f8f8bf16_rowwise_grouped_dynamic": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor zero_start_index_M, bool zeroing_output_tensor=True) -> Tensor",
     "f8f8bf16_rowwise_grouped_mm": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? offsets, Tensor(a!) output) -> Tensor",
     "f8f8bf16_rowwise_batched": "(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, Tensor? bias=None, bool use_fast_accum=True, Tensor(a!)? output=None) -> Tensor",
+    # no counterpart in the reference: its quantize_fp8_row -> f8f8bf16_rowwise pair as one operator (one launch at decode sizes)
+    "quantize_f8f8bf16_rowwise": "(Tensor X, Tensor WQ, Tensor w_scale, Tensor? bias=None) -> (Tensor, Tensor, Tensor)",
 }
 
 _library = torch.library.Library("mslk", "FRAGMENT")
@@ -148,6 +150,41 @@ def f8f8bf16_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
 
 def f8f8bf16_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_accum=True):
     _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output)
+
+
+def quantize_f8f8bf16_rowwise(X, WQ, w_scale, bias=None):
+    """bf16 activations in, bf16 out: `quantize_fp8_row(X, use_triton=False)` followed by `f8f8bf16_rowwise`, returning
+    (Y, XQ, x_scale) -- the pair every decode step of a caller of the reference issues (bench/gemm/gemm_ops.py:593-673).
+    For 1 <= M <= 4 rows of bf16 with K % 1024 == 0 it is ONE launch (every workgroup quantizes the rows itself; XQ and
+    x_scale are the bits the stand-alone quantizer returns); other shapes run the two kernels."""
+    _check(WQ.dtype == FP8_DTYPE, f"WQ must be {FP8_DTYPE} on gfx950, got {WQ.dtype}")
+    _check(w_scale.dtype == torch.float32, "Scales must be float32.")
+    _check(X.is_cuda and WQ.is_cuda and WQ.is_contiguous() and WQ.dim() == 2, "WQ must be a contiguous 2-D GPU tensor")
+    _check(X.dim() >= 1 and X.shape[-1] == WQ.shape[1], f"X and WQ must share K, got {X.shape[-1]} vs {WQ.shape[1]}")
+    N, K = WQ.shape
+    M = 1
+    for d in X.shape[:-1]:
+        M *= d
+    _check(w_scale.numel() == N, f"w_scale must have N={N} elements, got {w_scale.numel()}")
+    _check(w_scale.device == X.device and WQ.device == X.device, "all operands must be on the same device")
+    L = _lib.lib()
+    x2 = X.reshape(M, K) if M else X
+    one_launch = (X.dtype == torch.bfloat16 and M > 0 and L.mslk_amd_quantize_f8f8bf16_rowwise_supported(M, N, K)
+                  and x2.stride(-1) == 1 and x2.stride(0) % 8 == 0 and x2.data_ptr() % 16 == 0 and WQ.data_ptr() % 16 == 0)
+    if not one_launch:
+        from .quantize import quantize_fp8_row
+        XQ, x_scale = quantize_fp8_row(X, use_triton=False)
+        return _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, True), XQ, x_scale
+    ws = w_scale.contiguous()
+    bias_ptr, bias_code, _keep = _bias_args(bias, N, X.device)
+    Y = torch.empty(tuple(X.shape[:-1]) + (N,), dtype=torch.bfloat16, device=X.device)
+    XQ = torch.empty(X.shape, dtype=FP8_DTYPE, device=X.device)
+    x_scale = torch.empty(X.shape[:-1], dtype=torch.float32, device=X.device)
+    with _on_device(X.device):
+        _lib.check(L.mslk_amd_quantize_f8f8bf16_rowwise(
+            x2.data_ptr(), 0, x2.stride(0), WQ.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(), M, N, K,
+            XQ.data_ptr(), x_scale.data_ptr(), _stream_ptr(X.device)))
+    return Y, XQ, x_scale
 
 
 def f8f8f16_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
@@ -451,7 +488,14 @@ _IMPLS = {
     "f8f8bf16_rowwise_grouped_dynamic": f8f8bf16_rowwise_grouped_dynamic,
     "f8f8bf16_rowwise_grouped_mm": f8f8bf16_rowwise_grouped_mm,
     "f8f8bf16_rowwise_batched": f8f8bf16_rowwise_batched,
+    "quantize_f8f8bf16_rowwise": quantize_f8f8bf16_rowwise,
 }
+
+
+def _fake_quantize_rowwise(X, WQ, w_scale, bias=None):
+    return (torch.empty(tuple(X.shape[:-1]) + (WQ.shape[0],), dtype=torch.bfloat16, device=X.device),
+            torch.empty(X.shape, dtype=FP8_DTYPE, device=X.device),
+            torch.empty(X.shape[:-1], dtype=torch.float32, device=X.device))
 
 
 def _fake_rowwise(XQ, WQ, x_scale, w_scale, bias=None, use_fast_accum=True):
@@ -513,6 +557,7 @@ _FAKES = {
     "f8f8bf16_rowwise_grouped_dynamic": _fake_grouped_dynamic,
     "f8f8bf16_rowwise_grouped_mm": _fake_grouped_mm,
     "f8f8bf16_rowwise_batched": _fake_batched,
+    "quantize_f8f8bf16_rowwise": _fake_quantize_rowwise,
 }
 
 

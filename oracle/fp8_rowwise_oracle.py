@@ -205,6 +205,10 @@ def grouped_matmul_fp8_row_cpu(xq, wq, x_scale, w_scale) -> List[torch.Tensor]:
 # ----------------------------------------------------------------------------------------
 MAX_REL_TOL = 1e-2
 NORMWISE_TOL = 2e-3
+# elementwise criterion, as the reference's own tests compare (test/gemm/gemm_test.py:493-505,
+# test/gemm/triton/fp8_gemm_test.py:128-142), at the tolerance of the path: |y - ref| <= ELEM_RTOL * |ref| + ELEM_ATOL_RMS * rms(ref)
+ELEM_RTOL = 1e-2
+ELEM_ATOL_RMS = 1e-2
 
 
 def gemm_errors(y: torch.Tensor, ref: torch.Tensor) -> Tuple[float, float]:
@@ -219,3 +223,20 @@ def gemm_errors(y: torch.Tensor, ref: torch.Tensor) -> Tuple[float, float]:
     max_rel = diff.abs().max().item() / denom_max if denom_max > 0 else diff.abs().max().item()
     normwise = torch.linalg.vector_norm(diff).item() / denom_f if denom_f > 0 else torch.linalg.vector_norm(diff).item()
     return max_rel, normwise
+
+
+def gemm_elementwise_violations(y: torch.Tensor, ref: torch.Tensor, rms: float = None) -> Tuple[int, float]:
+    """Number of elements with |y - ref| > ELEM_RTOL * |ref| + ELEM_ATOL_RMS * rms(ref), and the largest value of
+    |y - ref| / (ELEM_RTOL * |ref| + ELEM_ATOL_RMS * rms(ref)) (<= 1 passes).  `rms` overrides rms(ref) when `ref`
+    is a block of a larger tensor."""
+    y64 = y.detach().cpu().to(torch.float64)
+    r64 = ref.detach().cpu().to(torch.float64)
+    if r64.numel() == 0:
+        return 0, 0.0
+    if rms is None:
+        rms = torch.sqrt(torch.mean(r64 * r64)).item()
+    bound = ELEM_RTOL * r64.abs() + ELEM_ATOL_RMS * rms
+    diff = (y64 - r64).abs()
+    bad = diff > bound
+    worst = (diff / bound.clamp_min(1e-300)).max().item() if rms > 0 else (0.0 if not bad.any() else float("inf"))
+    return int(bad.sum().item()), worst

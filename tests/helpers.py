@@ -39,8 +39,10 @@ def assert_quant_bit_exact(a_cpu: torch.Tensor, xq_gpu: torch.Tensor, scale_gpu:
     assert scale_gpu.shape == a_cpu.shape[:-1]
 
 
-def assert_gemm_close(y_gpu: torch.Tensor, ref: torch.Tensor, what: str = ""):
-    """north_star tolerance: max|y-ref|/max|ref| <= 1e-2 and ||y-ref||_F/||ref||_F <= 2e-3.
+def assert_gemm_close(y_gpu: torch.Tensor, ref: torch.Tensor, what: str = "", rms: float = None):
+    """north_star tolerance: max|y-ref|/max|ref| <= 1e-2 and ||y-ref||_F/||ref||_F <= 2e-3, plus the elementwise form the
+    reference's own tests use (test/gemm/gemm_test.py:493-505): |y-ref| <= 1e-2 |ref| + 1e-2 rms(ref) for EVERY element,
+    which a wrong small output element cannot hide behind a large one.
 
     One correct bf16 rounding alone costs up to 2^-8 relative per element (about 1.1e-3 normwise on
     average), so for outputs of fewer than 4096 elements -- where the norm does not average it out --
@@ -51,4 +53,6 @@ def assert_gemm_close(y_gpu: torch.Tensor, ref: torch.Tensor, what: str = ""):
     max_rel, normwise = O.gemm_errors(y_gpu.float(), ref)
     assert max_rel <= O.MAX_REL_TOL, f"{what}: max-rel {max_rel:.3e} > {O.MAX_REL_TOL}"
     assert normwise <= O.NORMWISE_TOL, f"{what}: normwise {normwise:.3e} > {O.NORMWISE_TOL}"
+    bad, worst = O.gemm_elementwise_violations(y_gpu.float(), ref, rms)
+    assert bad == 0, f"{what}: {bad} elements beyond rtol {O.ELEM_RTOL} / atol {O.ELEM_ATOL_RMS} rms (worst {worst:.2f} x the bound)"
     return max_rel, normwise

@@ -8,7 +8,7 @@ import mslk_amd
 from mslk_amd import workloads as W
 from oracle import c_twin
 from oracle import fp8_rowwise_oracle as O
-from tests.helpers import assert_gemm_close
+from tests.helpers import assert_gemm_close, assert_quant_bit_exact
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -274,7 +274,15 @@ def test_cfg2_full_with_bias():
     y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws, bias=bias)
     torch.cuda.synchronize()
     assert y.shape == (8192, 28672)
-    _check_sampled(y, xq, wq, xs, ws, bias, g, rows=64, what="cfg2")
+    # the WHOLE output against the fp32 oracle, in blocks of 1024 rows (1.9 TFLOP of CPU work in all): every tile, every
+    # tile edge and every pass of the persistent workgroups is covered, not a sample of rows
+    wq_c, ws_c, bias_c = wq.cpu(), ws.cpu(), bias.float().cpu()
+    wd = wq_c.float() * ws_c[:, None]                      # dequantized once
+    for r0 in range(0, 8192, 1024):
+        rows = slice(r0, r0 + 1024)
+        ref = (xq[rows].cpu().float() * xs[rows].cpu()[:, None]) @ wd.t() + bias_c[None, :]
+        assert_gemm_close(y[rows], ref, f"cfg2 rows {r0}..{r0 + 1023}")
+    del wd
     # linearity in the scales (size-independent property): doubling x_scale doubles y - bias exactly in fp32,
     # so the two bf16 outputs differ by at most one rounding
     y2 = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs * 2, ws, bias=bias)
@@ -295,7 +303,13 @@ def test_cfg3_decode(M):
     assert torch.equal(xq.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs.cpu().view(torch.int32), rs.view(torch.int32))
     y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
     torch.cuda.synchronize()
-    assert_gemm_close(y, O.dequant_matmul(rq, wq.cpu(), rs, ws.cpu()), f"cfg3 M={M}")
+    ref = O.dequant_matmul(rq, wq.cpu(), rs, ws.cpu())
+    assert_gemm_close(y, ref, f"cfg3 M={M}")
+    # the same step as ONE operator (one launch for M <= 4): quantized on the fly, same codes and scales, same tolerance
+    y1, xq1, xs1 = torch.ops.mslk.quantize_f8f8bf16_rowwise(x.to(DEV), wq, ws)
+    torch.cuda.synchronize()
+    assert torch.equal(xq1.cpu().view(torch.uint8), rq.view(torch.uint8)) and torch.equal(xs1.cpu().view(torch.int32), rs.view(torch.int32))
+    assert_gemm_close(y1, ref, f"cfg3 M={M}, quantizer fused")
 
 
 @pytest.mark.parametrize("M,N,K", [(512, 512, 256), (300, 260, 384), (16, 512, 512), (40, 300, 1040), (33, 20, 50),
@@ -475,3 +489,56 @@ def test_matches_the_model_level_fake_quant_statement(M, N, K):
     assert (err <= stated.float().abs() * 2.0 ** -7 + stated.float().abs().max() * 2.0 ** -10).all()
     max_rel, normwise = O.gemm_errors(y.float().cpu(), stated.float())
     assert max_rel <= O.MAX_REL_TOL and normwise <= 2 * O.NORMWISE_TOL
+
+
+@pytest.mark.parametrize("M,N,K,bias_dtype", [(1, 512, 1024, None), (3, 1000, 2048, torch.bfloat16), (4, 8200, 5120, torch.float32),
+                                              (2, 48, 3072, None), (4, 16, 8192, torch.bfloat16), (2, 4096, 14336, None),
+                                              (1, 520, 15360, None), (3, 300, 16384, None),
+                                              (7, 520, 2048, None), (4, 300, 1040, torch.bfloat16)])   # the last two: two launches
+def test_quantize_fused_into_the_decode_gemm(M, N, K, bias_dtype):
+    """quantize_f8f8bf16_rowwise: codes and scales are the stand-alone quantizer's bits (checked against the oracle),
+    the product meets the GEMM tolerance; rows of zeros, a NaN and an infinity behave as in the quantizer; the
+    activations may be a strided view."""
+    g = torch.Generator().manual_seed(M * 1000003 + N * 101 + K)
+    base = torch.randn(M, K + 24, generator=g).bfloat16()
+    x = base[:, 8:8 + K]                                   # row stride K + 24 elements, 16-byte aligned rows
+    if M >= 3:
+        x[1].zero_()
+    if M >= 4:
+        x[2, 17] = float("nan")
+        x[3, 100] = float("inf")
+    w = (torch.randn(N, K, generator=g) * 0.02).bfloat16()
+    wq, ws = O.quantize_fp8_row(w)
+    bias = None if bias_dtype is None else (torch.randn(N, generator=g) * 0.05).to(bias_dtype)
+    xd = base.to(DEV)[:, 8:8 + K]
+    y, xq, xs = torch.ops.mslk.quantize_f8f8bf16_rowwise(xd, wq.to(DEV), ws.to(DEV), None if bias is None else bias.to(DEV))
+    torch.cuda.synchronize()
+    assert y.shape == (M, N) and y.dtype == torch.bfloat16 and xq.shape == (M, K) and xs.shape == (M,)
+    assert_quant_bit_exact(x.contiguous(), xq, xs)
+    rq, rs = O.quantize_fp8_row(x.contiguous())
+    finite = torch.isfinite(rs) & ~torch.isnan(rq.float()).any(dim=1)
+    ref = O.dequant_matmul(rq[finite], wq, rs[finite], ws, None if bias is None else bias.float())
+    assert_gemm_close(y[finite.to(DEV)], ref, f"fused {M}x{N}x{K}")
+    if (~finite).any():
+        assert torch.isnan(y[(~finite).to(DEV)].float()).any(dim=1).all()
+
+
+def test_quantize_fused_graph_capture():
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(4, 4096, generator=g).bfloat16().to(DEV)
+    wq, ws = mslk_amd.quantize_fp8_row((torch.randn(1024, 4096, generator=g) * 0.02).bfloat16().to(DEV), use_triton=False)
+    eager = torch.ops.mslk.quantize_f8f8bf16_rowwise(x, wq, ws)[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        torch.ops.mslk.quantize_f8f8bf16_rowwise(x, wq, ws)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y, q, s = torch.ops.mslk.quantize_f8f8bf16_rowwise(x, wq, ws)
+    for _ in range(3):
+        y.fill_(7.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager)

@@ -112,13 +112,15 @@ def test_cfg4_full():
     ys = torch.ops.mslk.f8f8bf16_rowwise_grouped(xq, wq, xs, ws)
     torch.cuda.synchronize()
     assert sum(y.shape[0] for y in ys) == 8192
+    # every row of every expert against the fp32 oracle (0.69 TFLOP of CPU work): the ragged last tile of each expert,
+    # its last row and the tile edges of the large experts included
     for e, y in enumerate(ys):
         m = wl.counts[e]
+        assert y.shape == (m, 8192)
         if m == 0:
             continue
-        idx = torch.randperm(m, generator=g)[: min(8, m)]
-        ref = O.dequant_matmul(xq[e][idx.to(DEV)].cpu(), wq[e].cpu(), xs[e][idx.to(DEV)].cpu(), ws[e].cpu())
-        assert_gemm_close(y[idx.to(DEV)], ref, f"cfg4 expert {e}")
+        ref = O.dequant_matmul(xq[e].cpu(), wq[e].cpu(), xs[e].cpu(), ws[e].cpu())
+        assert_gemm_close(y, ref, f"cfg4 expert {e} ({m} rows)")
     # stacked entry point on the same data gives the same bits
     y2 = torch.ops.mslk.f8f8bf16_rowwise_grouped_stacked(xq_all, torch.stack(wq), xs_all, torch.stack(ws),
                                                          torch.tensor(wl.counts, dtype=torch.int64, device=DEV))

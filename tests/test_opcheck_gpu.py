@@ -27,6 +27,15 @@ def test_opcheck_quantize_and_dequantize():
     torch.library.opcheck(torch.ops.mslk.dequantize_fp8_row, (q, s), test_utils=CHECKS)
 
 
+def test_opcheck_quantize_fused_gemm():
+    x = torch.randn(5, 2048, device=DEV, dtype=torch.bfloat16)
+    torch.library.opcheck(torch.ops.mslk.quantize_f8f8bf16_rowwise, (x, _codes(96, 2048), torch.rand(96, device=DEV) + 0.5),
+                          test_utils=CHECKS)
+    x = torch.randn(40, 256, device=DEV, dtype=torch.bfloat16)       # two-launch shape
+    torch.library.opcheck(torch.ops.mslk.quantize_f8f8bf16_rowwise,
+                          (x, _codes(96, 256), torch.rand(96, device=DEV) + 0.5, torch.randn(96, device=DEV)), test_utils=CHECKS)
+
+
 def test_opcheck_dense_family():
     M, N, K = 80, 96, 256
     xq, wq = _codes(M, K), _codes(N, K)

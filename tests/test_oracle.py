@@ -359,3 +359,18 @@ def test_triton_arithmetic_closed_forms():
     assert torch.allclose(s1, s2, rtol=3e-7, atol=0)
     diff = (q1.view(torch.uint8).int() - q2.view(torch.uint8).int()).abs()
     assert diff.max() <= 1 and (diff != 0).float().mean() < 1e-2
+
+
+def test_elementwise_criterion_counts_what_it_should():
+    ref = torch.tensor([[100.0, -100.0, 0.0, 1.0]], dtype=torch.float32)      # rms = sqrt(20001 / 4) = 70.71
+    assert O.gemm_elementwise_violations(ref.clone(), ref) == (0, 0.0)
+    y = ref.clone()
+    y[0, 0] = 101.7                      # bound 1e-2 * 100 + 1e-2 * 70.71 = 1.707: just inside
+    y[0, 2] = 0.70                       # bound 0.7071: inside
+    assert O.gemm_elementwise_violations(y, ref)[0] == 0
+    y[0, 1] = -101.8                     # beyond 1.707
+    y[0, 3] = 1.8                        # |diff| 0.8 > 1e-2 + 0.7071
+    bad, worst = O.gemm_elementwise_violations(y, ref)
+    assert bad == 2 and abs(worst - 0.8 / (0.01 + 0.70712)) < 1e-3
+    # a block of a larger tensor: the caller's rms replaces the block's own
+    assert O.gemm_elementwise_violations(y, ref, rms=1000.0)[0] == 0
