@@ -18,11 +18,12 @@
 //   * Two XQ buffers and three WQ buffers: while step k is multiplied, the XQ tile of step k+1 and the
 //     WQ tiles of steps k+1 and k+2 are in flight (the weights are the cold, read-once stream).
 // Rows
-//   * The 16-row m fragments of a tile are dealt to the wave rows round-robin (wave row wm owns fragments wm, wm + WM,
-//     ...).  With ROWSKIP a tile with fewer valid rows than BM runs a K loop compiled for a quarter, half or three
-//     quarters of the m fragments per wave and leaves out the XQ loads and the epilogue work of fragments without valid
-//     rows: the cost of a ragged tile (the last row tile of an MoE group) follows its row count in steps of BM / 4 rows,
-//     down to what the weight stream alone costs.
+//   * A wave row owns BM / WM consecutive rows of a tile.  With ROWSKIP (the grouped kernels) a tile with at most three
+//     quarters of its rows valid is multiplied differently: its 16-row m fragments are dealt to the wave rows round-robin
+//     (wave row wm owns fragments wm, wm + WM, ...), the K loop is one compiled for a quarter, half or three quarters of
+//     the m fragments per wave, and the XQ loads and the epilogue work of fragments without valid rows are left out: the
+//     cost of a ragged tile (the last row tile of an MoE group) follows its row count in steps of BM / 4 rows, down to
+//     what the weight stream alone costs.  (Dealing the fragments of FULL tiles round-robin as well cost 2 % on them.)
 // Math
 //   * v_mfma_f32_16x16x128_f8f6f4 (both operands e4m3, unit block scales).  WQ rows are the first
 //     operand and XQ rows the second, so a lane ends up holding 4 consecutive n for one m.
@@ -199,8 +200,11 @@ struct GemmTile {
     const v4i hi = *reinterpret_cast<const v4i*>(tile + t * STRIDE + fo.off1);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   }
-  static constexpr int A_FRAG_STRIDE = TS::WM * 16 * kBK;   // wave row wm owns the m fragments wm, wm + WM, ...
-  MSLK_AMD_DEVINL static v8i load_frag_a(const char* tile, int t, FragOff fo) { return load_frag<A_FRAG_STRIDE>(tile, t, fo); }
+  // ILV (ragged tiles): wave row wm owns the m fragments wm, wm + WM, ...; otherwise the fragments wm * FM ... wm * FM + FM - 1
+  template <bool ILV>
+  MSLK_AMD_DEVINL static v8i load_frag_a(const char* tile, int t, FragOff fo) {
+    return load_frag<(ILV ? TS::WM : 1) * 16 * kBK>(tile, t, fo);
+  }
   // WQ fragment t of the wave: as load_frag, or lane-linear out of the two 1 KiB blocks of row group t.
   MSLK_AMD_DEVINL static v8i load_frag_b(const char* tile, int t, FragOff fo) {
     if constexpr (PS) {
@@ -213,8 +217,9 @@ struct GemmTile {
     }
   }
   // The part of an XQ / WQ buffer this wave multiplies.
+  template <bool ILV = false>
   MSLK_AMD_DEVINL static const char* a_tile_of(const char* abuf) {
-    return abuf + (wave_id() / TS::WN) * 16 * kBK;
+    return abuf + (wave_id() / TS::WN) * (ILV ? 16 : TS::kBM / TS::WM) * kBK;
   }
   MSLK_AMD_DEVINL static const char* b_tile_of(const char* bbuf) {
     return bbuf + (wave_id() % TS::WN) * (TS::kBN / TS::WN) * kBK;
@@ -225,7 +230,7 @@ struct GemmTile {
     const FragOff fo = frag_off();
     wf0 = load_frag_b(b_tile_of(bbuf), 0, fo);
 #pragma unroll
-    for (int tm = 0; tm < FMV; ++tm) xf[tm] = load_frag_a(a_tile_of(abuf), tm, fo);
+    for (int tm = 0; tm < FMV; ++tm) xf[tm] = load_frag_a<(FMV < TS::FM)>(a_tile_of<(FMV < TS::FM)>(abuf), tm, fo);
   }
 
   // Waits until at most `pending` of this wave's DMA loads (the youngest ones) are still in flight and
@@ -309,12 +314,12 @@ struct GemmTile {
       wait_and_barrier<PENDING>();
       wf0 = load_frag_b(b_tile_of(b_nxt), 0, fo);
     }
-    const char* a_next = a_tile_of(a_nxt);
+    const char* a_next = a_tile_of<false>(a_nxt);
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
       acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
       if constexpr (NEXT) {
-        xf[tm] = load_frag_a(a_next, tm, fo);
+        xf[tm] = load_frag_a<false>(a_next, tm, fo);
         __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
       }
     }
@@ -351,12 +356,12 @@ struct GemmTile {
       wait_and_barrier<PENDING>();
       wf0 = load_frag_b(b_tile_of(b_nxt), 0, fo);
     }
-    const char* a_next = a_tile_of(a_nxt);
+    const char* a_next = a_tile_of<true>(a_nxt);
 #pragma unroll
     for (int tm = 0; tm < FMV; ++tm) {
       acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
       if constexpr (NEXT) {
-        xf[tm] = load_frag_a(a_next, tm, fo);
+        xf[tm] = load_frag_a<true>(a_next, tm, fo);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
@@ -534,6 +539,19 @@ struct GemmTile {
     const bool full = n_rem >= TS::kBN && vec16 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
                       (BIAS == 0 || (reinterpret_cast<uintptr_t>(bias) & (BIAS == 1 ? 15 : 7)) == 0);
     const bool interior = full && m_rem >= TS::kBM;   // no bounds logic at all
+    if constexpr (ROWSKIP && TS::RING == 0 && TS::FM % 4 == 0) {
+      // a tile multiplied by one of the reduced K loops has its m fragments dealt to the wave rows round-robin
+      if (m_rem <= 3 * (TS::kBM / 4)) {
+        if (out_f16) {
+          if (full) epilogue_impl<true, true, false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+          else epilogue_impl<false, true, false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+        } else {
+          if (full) epilogue_impl<true, false, false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+          else epilogue_impl<false, false, false, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
+        }
+        return;
+      }
+    }
     if (out_f16) {
       if (interior) epilogue_impl<true, true, true>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
       else if (full) epilogue_impl<true, true, false>(buf, acc, xs, ws, bias, y, m_rem, n_rem, N);
@@ -547,7 +565,8 @@ struct GemmTile {
 
   // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged unless
   // ALL_ROWS says that the tile has all its rows too.
-  template <bool FULL, bool F16, bool ALL_ROWS>
+  // ILV: the m fragments of the tile were dealt to the wave rows round-robin (ragged tiles of the grouped kernels).
+  template <bool FULL, bool F16, bool ALL_ROWS, bool ILV = false>
   MSLK_AMD_DEVINL void epilogue_impl(char* buf, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
                                      const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
     constexpr int WN = TS::kBN / TS::WN;         // columns per wave
@@ -565,14 +584,14 @@ struct GemmTile {
     constexpr int ROWS_W = TS::kBM / TS::WM;     // rows per wave
     static_assert(2 * BUF + ROWS_W * 4 == EPI_WAVE_BYTES, "epilogue buffer size");
     const int n_base = wn * WN;
-    // tile row of row j of this wave's m fragment tm (the fragments of a tile are dealt to the wave rows round-robin)
-    auto frag_row = [&](int tm) { return (tm * TS::WM + wm) * 16; };
+    // tile row of row 0 of this wave's m fragment tm
+    auto frag_row = [&](int tm) { return ILV ? (tm * TS::WM + wm) * 16 : wm * (TS::kBM / TS::WM) + tm * 16; };
     // fragments of this wave with at least one valid row (formed from m_rem: a persistent workgroup has already run
     // init() for its next tile when the epilogue of the current one starts)
     int fm_live = TS::FM;
     if constexpr (!ALL_ROWS) {
       const int nf = ((m_rem < TS::kBM ? m_rem : TS::kBM) + 15) >> 4;
-      const int mine = (nf - wm + TS::WM - 1) / TS::WM;
+      const int mine = ILV ? (nf - wm + TS::WM - 1) / TS::WM : nf - wm * TS::FM;
       fm_live = mine < 0 ? 0 : (mine > TS::FM ? TS::FM : mine);
     }
     const bool vec_store = (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
@@ -676,7 +695,7 @@ struct GemmTile {
       // one 64-bit add per store
       char* dst = reinterpret_cast<char*>(y + (int64_t)frag_row(0) * N) + lane_off;
       const int64_t dst_step = (int64_t)RPI * N * 2;
-      const int64_t frag_step = (int64_t)(TS::WM - 1) * 16 * N * 2;
+      const int64_t frag_step = ILV ? (int64_t)(TS::WM - 1) * 16 * N * 2 : 0;
       float xsv = xs_lds[j];
 #pragma unroll
       for (int tm = 0; tm <= TS::FM; ++tm) {
@@ -698,7 +717,7 @@ struct GemmTile {
           }
           __builtin_amdgcn_sched_barrier(0);
         }
-        if (tm > 0 && TS::WM > 1) dst += frag_step;
+        if (ILV && tm > 0 && TS::WM > 1) dst += frag_step;
         xsv = xsv_next;
       }
     } else {
