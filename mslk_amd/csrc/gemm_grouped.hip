@@ -99,56 +99,92 @@ MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
     }
   } else {
     // The G extents are read 64 at a time, one per lane, and turned into tile ranges by a wave-level
-    // prefix sum, so the lookup costs one memory round trip instead of G dependent ones.
+    // prefix sum, so the lookup costs one memory round trip instead of G dependent ones.  The total tile count is formed
+    // first: XCD x (workgroup id mod 8) then takes a contiguous slice of the tile list, so that the row tiles of a group
+    // that share a weight panel run on one XCD and find it in its L2 (without the slices the device-extent layouts
+    // fetched 1.6 times what the host-extent kernel fetches for the same 16 experts).
     const int fixed_tiles = LAYOUT == kGroupsOffsetsN ? tiles_m : tiles_n;
     const int blk = LAYOUT == kGroupsOffsetsN ? BN : BM;
     const int64_t total = LAYOUT == kGroupsOffsetsN ? p.N : p.M;
     const int lane = threadIdx.x & 63;
-    int64_t carry_tiles = 0, carry_len = 0;
-    for (int base = 0; base < p.G; base += 64) {
+    // Every quantity fits 32 bits (the host checks the dimensions and the grid): sizes beyond the tensor mark the group bad.
+    struct Chunk { int start, len, tiles, incl; bool bad; };
+    auto load_chunk = [&](int base, int& carry_len) {
+      Chunk c;
       const int gi = base + lane;
       const bool in = gi < p.G;
-      int64_t start = 0, len = 0;
+      c.start = 0;
+      c.len = 0;
+      c.bad = false;
       if constexpr (LAYOUT == kGroupsSizesM) {
-        if (in) len = static_cast<const int64_t*>(p.layout)[gi];
-        int64_t incl_len = len;
+        int64_t len64 = 0;
+        if (in) len64 = static_cast<const int64_t*>(p.layout)[gi];
+        c.bad = len64 < 0 || len64 > total;
+        c.len = c.bad ? 0 : (int)len64;
+        // running sum that saturates at 2^31 - 1 instead of wrapping (the terms are below 2^31, so one unsigned addition
+        // cannot wrap): sizes that add up to more than the tensor holds always end beyond it and mark their group bad
+        auto sat_add = [](int x, int y) {
+          const uint32_t u = (uint32_t)x + (uint32_t)y;
+          return (int)(u > 0x7FFFFFFFu ? 0x7FFFFFFFu : u);
+        };
+        int incl_len = c.len;
 #pragma unroll
         for (int d = 1; d < 64; d <<= 1) {
-          const int64_t v = __shfl_up(incl_len, d, 64);
-          if (lane >= d) incl_len += v;
+          const int v = __shfl_up(incl_len, d, 64);
+          if (lane >= d) incl_len = sat_add(incl_len, v);
         }
-        start = carry_len + incl_len - len;
-        carry_len += __shfl(incl_len, 63, 64);
+        const int end = sat_add(carry_len, incl_len);
+        c.start = end - c.len;
+        carry_len = sat_add(carry_len, __shfl(incl_len, 63, 64));
+        c.bad = c.bad || (in && (end > total || end == 0x7FFFFFFF));
       } else {
         const int32_t* off = static_cast<const int32_t*>(p.layout);
         if (in) {
-          start = gi ? off[gi - 1] : 0;
-          len = (int64_t)off[gi] - start;
+          c.start = gi ? off[gi - 1] : 0;
+          const int64_t len64 = (int64_t)off[gi] - c.start;
+          c.bad = len64 < 0 || c.start < 0 || (int64_t)c.start + len64 > total;
+          c.len = c.bad ? 0 : (int)len64;
         }
       }
-      const bool bad = in && (len < 0 || start < 0 || start + len > total);   // inconsistent group data
-      const int64_t tiles = (in && !bad) ? ((len + blk - 1) / blk) * fixed_tiles : 0;
-      int64_t incl = tiles;
+      c.tiles = (in && !c.bad) ? ((c.len + blk - 1) / blk) * fixed_tiles : 0;
+      c.incl = c.tiles;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
-        const int64_t v = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += v;
+        const int v = __shfl_up(c.incl, d, 64);
+        if (lane >= d) c.incl += v;
       }
-      const int64_t excl = carry_tiles + incl - tiles;
-      const bool hit = tiles > 0 && t >= excl && t < excl + tiles;
-      const unsigned long long hit_mask = __ballot(hit), bad_mask = __ballot(bad);
+      return c;
+    };
+    int64_t total_tiles = 0;
+    int carry_len = 0;
+    Chunk first = load_chunk(0, carry_len);
+    total_tiles = __shfl(first.incl, 63, 64);
+    for (int base = 64; base < p.G; base += 64) total_tiles += __shfl(load_chunk(base, carry_len).incl, 63, 64);
+    const int64_t per_xcd = (total_tiles + kXcds - 1) / kXcds;
+    const int64_t slot = t / kXcds;                       // `t` arrives as the workgroup id
+    const int64_t tile = (int64_t)(t % kXcds) * per_xcd + slot;
+    if (slot >= per_xcd || tile >= total_tiles) return false;
+    int64_t carry_tiles = 0;
+    carry_len = 0;
+    for (int base = 0; base < p.G; base += 64) {
+      Chunk c = first;
+      if (base == 0) carry_len = __shfl(first.start + first.len, 63, 64);   // sizes: rows of the first 64 groups
+      else c = load_chunk(base, carry_len);
+      const int64_t excl = carry_tiles + c.incl - c.tiles;
+      const bool hit = c.tiles > 0 && tile >= excl && tile < excl + c.tiles;
+      const unsigned long long hit_mask = __ballot(hit), bad_mask = __ballot(c.bad);
       if (hit_mask != 0) {
         const int src = __ffsll((long long)hit_mask) - 1;
         if (bad_mask & ((1ull << src) - 1ull)) return false;   // a group before this one is inconsistent: touch nothing
         // the results are the same in every lane: say so, so that the tile's addresses live in scalar registers
         sp.gi = base + src;
-        sp.o0 = uniform64(__shfl(start, src, 64));
-        sp.len = __builtin_amdgcn_readfirstlane((int)__shfl(len, src, 64));
-        sp.t = t - __builtin_amdgcn_readfirstlane((int)__shfl(excl, src, 64));
+        sp.o0 = __builtin_amdgcn_readfirstlane(__shfl(c.start, src, 64));
+        sp.len = __builtin_amdgcn_readfirstlane(__shfl(c.len, src, 64));
+        sp.t = (int)(tile - uniform64(__shfl(excl, src, 64)));
         return true;
       }
       if (bad_mask != 0) return false;
-      carry_tiles += __shfl(incl, 63, 64);
+      carry_tiles += __shfl(c.incl, 63, 64);
     }
     return false;
   }
@@ -239,9 +275,9 @@ hipError_t launch_device_shape(const DeviceGroups& p, hipStream_t s) {
   if (LAYOUT == kGroupsUniform || LAYOUT == kGroupsOffsetsK || LAYOUT == kGroupsPrepadM) {
     grid = (p.G * tiles_m * tiles_n + kXcds - 1) / kXcds * kXcds;
   } else if (LAYOUT == kGroupsOffsetsN) {
-    grid = tiles_m * (tiles_n + p.G);   // every group may end in a partial tile
+    grid = (tiles_m * (tiles_n + p.G) + kXcds - 1) / kXcds * kXcds;   // every group may end in a partial tile; 8 slices
   } else {
-    grid = (tiles_m + p.G) * tiles_n;
+    grid = ((tiles_m + p.G) * tiles_n + kXcds - 1) / kXcds * kXcds;
   }
   if (grid <= 0) return hipSuccess;
   if (grid > 2147483647) return hipErrorInvalidValue;

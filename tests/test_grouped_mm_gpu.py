@@ -169,6 +169,28 @@ def test_inconsistent_offsets_write_nothing_out_of_range():
     assert (out[64:] == SENTINEL).all()
 
 
+@pytest.mark.parametrize("sizes", [[64, 10000], [64, 2 ** 40], [64, -3, 20], [64] + [2 ** 30] * 4 + [32], [2 ** 31 - 1, 2 ** 31 - 1, 2]])
+def test_inconsistent_sizes_of_the_stacked_entry_point_write_nothing_out_of_range(sizes):
+    """int64 group sizes that do not fit the tensor (too large, negative, or adding up past 2^31 so that a 32-bit running sum
+    would wrap): groups before the first bad one are computed, nothing else is touched."""
+    from mslk_amd import _lib
+    g = torch.Generator().manual_seed(6)
+    M, N, K, G = 128, 512, 512, len(sizes)
+    xq, xs = _quant(M, K, g)
+    wq, ws = _quant(G * N, K, g, 0.02)
+    out = _sentinel(M, N)
+    dev = [t.to(DEV) for t in (xq, wq, xs, ws)]
+    msz = torch.tensor(sizes, dtype=torch.int64, device=DEV)
+    _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped_stacked(dev[0].data_ptr(), dev[1].data_ptr(), dev[2].data_ptr(),
+                                                                    dev[3].data_ptr(), msz.data_ptr(), G, M, N, K, out.data_ptr(),
+                                                                    torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    good = sizes[0] if 0 <= sizes[0] <= M else 0
+    if good:
+        assert_gemm_close(out[:good], O.dequant_matmul(xq[:good], wq[:N], xs[:good], ws[:N]))
+    assert (out[good:] == SENTINEL).all()
+
+
 def test_argument_checks_follow_the_reference():
     XQ = torch.zeros(64, 512, dtype=F8, device=DEV)
     WQ = torch.zeros(2, 512, 512, dtype=F8, device=DEV)
