@@ -75,8 +75,12 @@ MSLK_AMD_DEVINL uint32_t finish_absmax_bits(uint32_t m) {
 }
 
 // `factor` is the multiplier `inv` of the torch-branch formula, or the divisor `scale` of the Triton one.
+// TRITON with rcp != 0: x / factor is formed as q0 = x * rcp, e = fma(-q0, factor, x), q = e == 0 ? q0 : fma(e, rcp, q0)
+// with rcp = fl32(1 / factor) -- a handful of instructions instead of a division sequence.  The e4m3 codes are those of the
+// IEEE division for every 16-bit element not above a 16-bit row maximum of at least 2^-64 (checked exhaustively on the
+// CPU, tests/test_oracle.py); the caller passes rcp = 0 for every other row, which then divides.
 template <int DTYPE, bool TRITON>
-MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float factor) {
+MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float factor, float rcp = 0.f) {
   float f[8];
   if constexpr (DTYPE == 2) {
     const uint32_t w[8] = {v.lo.x, v.lo.y, v.lo.z, v.lo.w, v.hi.x, v.hi.y, v.hi.z, v.hi.w};
@@ -90,10 +94,22 @@ MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float factor) {
       f[2 * i + 1] = Traits<DTYPE>::to_f32(w[i] >> 16);
     }
   }
+  if constexpr (TRITON) {
+    if (rcp != 0.f) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    if constexpr (TRITON) f[i] = __builtin_fminf(__builtin_fmaxf(f[i] / factor, -448.0f), 448.0f);
-    else f[i] = f[i] * factor;
+      for (int i = 0; i < 8; ++i) {
+        const float q0 = f[i] * rcp;
+        const float e = __builtin_fmaf(-q0, factor, f[i]);
+        const float q = e == 0.f ? q0 : __builtin_fmaf(e, rcp, q0);
+        f[i] = __builtin_fminf(__builtin_fmaxf(q, -448.0f), 448.0f);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) f[i] = __builtin_fminf(__builtin_fmaxf(f[i] / factor, -448.0f), 448.0f);
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = f[i] * factor;
   }
   uint2 r;
   r.x = cvt_pk_e4m3fn(f[0], f[1]) | (cvt_pk_e4m3fn(f[2], f[3]) << 16);
@@ -137,6 +153,15 @@ MSLK_AMD_DEVINL uint32_t team_max(uint32_t m, uint32_t* smem, int team_in_block)
   return m;
 }
 
+// Reciprocal of the Triton-arithmetic divisor for rows that may use the multiply form of quantize_vec8, else 0: the row
+// maximum is a finite 16-bit value of at least 2^-64 that neither the lower bound nor scale_ub replaced.
+template <int DTYPE, bool TRITON>
+MSLK_AMD_DEVINL float triton_fast_rcp(float amax, const float* scale_ub, float triton_eps, float divisor) {
+  if constexpr (!TRITON || DTYPE == 2) return 0.f;
+  const bool ok = scale_ub == nullptr && amax >= triton_eps && amax >= 0x1p-64f && amax < __builtin_inff();
+  return ok ? 1.0f / divisor : 0.f;
+}
+
 // Vector path: K % 8 == 0, row starts 16-byte aligned, output rows 8-byte aligned.
 template <int DTYPE, int TEAM, int NV, bool CACHED, bool TRITON>
 __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
@@ -172,8 +197,10 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
   if (!valid) return;
 
   float inv, sc;
-  scales_from_amax<DTYPE, TRITON>(Traits<DTYPE>::abs_bits_to_f32(m), scale_ub, jag.triton_eps, inv, sc);
+  const float amax = Traits<DTYPE>::abs_bits_to_f32(m);
+  scales_from_amax<DTYPE, TRITON>(amax, scale_ub, jag.triton_eps, inv, sc);
   if (lane == 0) scale[row] = sc;
+  const float rcp = triton_fast_rcp<DTYPE, TRITON>(amax, scale_ub, jag.triton_eps, inv);
 
   uint2* out_row = reinterpret_cast<uint2*>(out + row * out_stride);
   if (!live) {   // an empty row quantizes to zero codes
@@ -182,11 +209,11 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = i * TEAM + lane;
-      if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(cache[i], inv));
+      if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(cache[i], inv, rcp));
     }
   } else {
     for (int idx = lane; idx < nvec; idx += TEAM)
-      store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(load_vec8<DTYPE>(row_ptr, idx), inv));
+      store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(load_vec8<DTYPE>(row_ptr, idx), inv, rcp));
   }
   // zero padding columns [K, out_stride)
   for (int64_t k = K + lane; k < out_stride; k += TEAM) out[row * out_stride + k] = 0;

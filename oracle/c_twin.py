@@ -37,8 +37,20 @@ def lib() -> ctypes.CDLL:
                                            ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
         L.oracle_dequant_gemm.restype = None
         L.oracle_dequant_gemm.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int64] * 3 + [ctypes.c_void_p]
+        L.oracle_count_division_mismatches.restype = ctypes.c_uint64
+        L.oracle_count_division_mismatches.argtypes = [ctypes.c_int, ctypes.c_uint32, ctypes.c_uint32,
+                                                       ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32)]
         _lib = L
     return _lib
+
+
+def count_division_mismatches(dtype: torch.dtype, first_c_bits: int = 0, end_c_bits: int = 0):
+    """Pairs (row maximum c, element x) of 16-bit values, c bits in [first_c_bits, end_c_bits), whose e4m3 code differs
+    between the IEEE division x / (c / 448) and the reciprocal + two fused multiply-adds the quantizer kernel uses.
+    Returns (count, first offending pair, last offending pair) with pairs as (c bits << 16 | x bits)."""
+    fb, lb = ctypes.c_uint32(0), ctypes.c_uint32(0)
+    n = lib().oracle_count_division_mismatches(_DTYPE_CODE[dtype], first_c_bits, end_c_bits, ctypes.byref(fb), ctypes.byref(lb))
+    return int(n), fb.value, lb.value
 
 
 def e4m3fn_cast(x: torch.Tensor) -> torch.Tensor:

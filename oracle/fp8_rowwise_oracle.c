@@ -153,3 +153,45 @@ void oracle_dequant_gemm(const uint8_t* xq, const uint8_t* wq, const float* xs, 
       y[m * N + n] = acc + (bias ? (double)bias[n] : 0.0);
     }
 }
+
+/*
+ * Checker for a kernel optimisation, not a restatement of the reference: the quantizer's Triton-arithmetic mode needs
+ * code = e4m3fn(clamp(x / s, -448, 448)) with an IEEE division (div_rn, mslk/quantize/triton/fp8_quantize.py:164-166),
+ * s = fl32(c / 448), for every element x of a row whose maximum is c.  The kernel replaces the division by
+ *     r = fl32(1 / s);  q0 = fl32(x * r);  e = fma(-q0, s, x);  q = e == 0 ? q0 : fma(e, r, q0)
+ * (a handful of instructions per element instead of a division sequence; rows whose r is not finite keep the division).
+ * This function walks EVERY pair (c, x) of 16-bit values of the given dtype (0 bf16, 1 fp16) with c finite and positive,
+ * r finite and |x| <= c, and counts the pairs whose code differs between the two forms; `first_bad` / `last_bad`
+ * receive the first and the last offending pair as (c bits << 16 | x bits); the walk covers c bits in
+ * [first_c_bits, end_c_bits) (0 = from the smallest / to the largest finite value).
+ */
+uint64_t oracle_count_division_mismatches(int dtype, uint32_t first_c_bits, uint32_t end_c_bits, uint32_t* first_bad,
+                                          uint32_t* last_bad) {
+  uint64_t bad = 0;
+  uint32_t top = dtype == 0 ? 0x7F80u : 0x7C00u;      /* first non-finite magnitude */
+  if (end_c_bits > 0 && end_c_bits < top) top = end_c_bits;
+  for (uint32_t cb = first_c_bits > 0 ? first_c_bits : 1; cb < top; ++cb) {
+    const float c = dtype == 0 ? bf16_to_f32((uint16_t)cb) : f16_to_f32((uint16_t)cb);
+    const float s = c / 448.0f;
+    const float r = 1.0f / s;
+    if (!(r <= 3.4028234663852886e38f)) continue;   /* r overflowed: the kernel divides in such rows */
+    for (uint32_t xb = 0; xb <= cb; ++xb) {
+      for (int sign = 0; sign < 2; ++sign) {
+        const uint16_t bits = (uint16_t)(xb | (sign ? 0x8000u : 0u));
+        const float x = dtype == 0 ? bf16_to_f32(bits) : f16_to_f32(bits);
+        float want = x / s;
+        const float q0 = x * r;
+        const float e = fmaf(-q0, s, x);
+        float got = e == 0.0f ? q0 : fmaf(e, r, q0);
+        want = want < -448.0f ? -448.0f : (want > 448.0f ? 448.0f : want);
+        got = got < -448.0f ? -448.0f : (got > 448.0f ? 448.0f : got);
+        if (oracle_e4m3fn_from_f32(want) != oracle_e4m3fn_from_f32(got)) {
+          if (bad == 0 && first_bad) *first_bad = (cb << 16) | bits;
+          if (last_bad) *last_bad = (cb << 16) | bits;
+          ++bad;
+        }
+      }
+    }
+  }
+  return bad;
+}
