@@ -11,6 +11,8 @@
 //     needed.  The batched op (csrc/gemm/ck/fp8_rowwise_batched/fp8_rowwise_batched_gemm.hip:199-254)
 //     is the uniform layout.
 // Empty groups own no tiles and are never touched.
+#include <algorithm>
+
 #include "gemm_tile.h"
 #include "kernels.h"
 
@@ -33,10 +35,10 @@ template <int BM, int BN>
 __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
   using TS = TileShape<BM, BN>;
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
-  // XCD x works on a contiguous slice of the tile list.
-  const int per_xcd = (tab.total_tiles + kXcds - 1) / kXcds;
-  const int t = (blockIdx.x % kXcds) * per_xcd + blockIdx.x / kXcds;
-  if (t >= tab.total_tiles) return;
+  // XCD x works on its own contiguous slice of the tile list (the launcher has cut the list by estimated cost).
+  const int xcd = blockIdx.x % kXcds;
+  const int t = tab.xcd_begin[xcd] + blockIdx.x / kXcds;
+  if (t >= tab.xcd_begin[xcd + 1]) return;
   // group lookup in one step: lane i compares against the first tile of group i (count <= 64, begins ascend)
   const int lane = threadIdx.x & 63;
   const int begin = lane < tab.count ? tab.g[lane].tile_begin : 0x7FFFFFFF;
@@ -301,10 +303,86 @@ hipError_t launch_device_layout(const DeviceGroups& p, hipStream_t s) {
 
 }  // namespace
 
-hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s) {
-  if (t.total_tiles <= 0) return hipSuccess;
-  const int grid = ((t.total_tiles + kXcds - 1) / kXcds) * kXcds;
-  grouped_tiled_kernel<256, 256><<<grid, 256, 0, s>>>(t);
+// Host-side schedule of a TensorList launch.  Workgroup ids go round the eight XCDs, and inside an XCD the hardware
+// hands the next workgroup to the first CU that is free -- so an XCD finishes when its share of the WORK is done, and
+// the launch when the slowest XCD is.  Equal tile COUNTS per XCD are not equal work: a tile of an expert with one row
+// tile fetches its whole weight block from HBM alone (measured about 67 us at K = 5120), a tile out of a panel of four
+// row tiles shares it (59 us), and a ragged tile with a quarter of the rows takes about three quarters of a full one.
+// The groups are therefore cut into panels of up to kGroupM row tiles (all column tiles of those rows: the unit inside
+// which operand tiles are shared through the L2), every panel gets a cost from that model, the panels are dealt to the
+// XCDs longest first onto the least loaded one, and inside an XCD the panels with the cheapest tiles come last, so
+// that the last pass over the CUs is a short one.  A panel is just another group descriptor (same weights, row range
+// of the activations and of the output); when the panels would not fit the descriptor table, whole groups are dealt.
+hipError_t launch_grouped_tiled(const GroupTable& in, hipStream_t s) {
+  if (in.total_tiles <= 0 || in.count <= 0) return hipSuccess;
+  constexpr int BM = 256, BN = 256;
+  struct Chunk { int group, row0, rows, tiles; float cost, cheapest; };
+  Chunk chunks[kMaxGroupsPerLaunch];
+  auto tile_cost = [](int rows, int sharing) {   // relative time of one tile: rows valid, `sharing` row tiles use its weights
+    const int q = (rows + BM / 4 - 1) / (BM / 4);
+    static const float base[5] = {0.f, 42.4f, 48.3f, 55.0f, 56.7f};
+    return base[q < 4 ? q : 4] + 9.3f / (float)sharing;
+  };
+  auto cut = [&](int rows_per_chunk) {   // number of chunks, or -1 if they do not fit
+    int n = 0;
+    for (int g = 0; g < in.count; ++g) {
+      const GroupDesc& d = in.g[g];
+      const int tiles_n = (d.N + BN - 1) / BN;
+      for (int64_t r0 = 0; r0 < d.M; r0 += rows_per_chunk) {
+        if (n == kMaxGroupsPerLaunch) return -1;
+        const int rows = (int)(d.M - r0 < rows_per_chunk ? d.M - r0 : rows_per_chunk);
+        const int tiles_m = (rows + BM - 1) / BM;
+        Chunk& c = chunks[n++];
+        c.group = g; c.row0 = (int)r0; c.rows = rows; c.tiles = tiles_m * tiles_n;
+        const int last = rows - (tiles_m - 1) * BM;
+        c.cheapest = tile_cost(last, tiles_m);
+        c.cost = (float)tiles_n * ((float)(tiles_m - 1) * tile_cost(BM, tiles_m) + c.cheapest);
+      }
+    }
+    return n;
+  };
+  int n = cut(kGroupM * BM);
+  if (n < 0) n = cut(0x7FFFFF00);   // one chunk per group always fits
+  // longest first onto the least loaded XCD
+  int order[kMaxGroupsPerLaunch];
+  for (int i = 0; i < n; ++i) order[i] = i;
+  std::stable_sort(order, order + n, [&](int a, int b) { return chunks[a].cost > chunks[b].cost; });
+  int bin_of[kMaxGroupsPerLaunch];
+  float load[kXcds] = {};
+  for (int i = 0; i < n; ++i) {
+    int best = 0;
+    for (int x = 1; x < kXcds; ++x)
+      if (load[x] < load[best]) best = x;
+    bin_of[order[i]] = best;
+    load[best] += chunks[order[i]].cost;
+  }
+  // inside an XCD: panels whose cheapest tile is expensive first
+  std::stable_sort(order, order + n, [&](int a, int b) {
+    if (bin_of[a] != bin_of[b]) return bin_of[a] < bin_of[b];
+    return chunks[a].cheapest > chunks[b].cheapest;
+  });
+  GroupTable t;
+  t.count = n;
+  int tiles = 0, longest = 0, x = 0;
+  t.xcd_begin[0] = 0;
+  for (int i = 0; i < n; ++i) {
+    const Chunk& c = chunks[order[i]];
+    while (x < bin_of[order[i]]) t.xcd_begin[++x] = tiles;
+    const GroupDesc& d = in.g[c.group];
+    GroupDesc& o = t.g[i];
+    o = d;
+    o.xq = d.xq + (int64_t)c.row0 * d.K;
+    o.xs = d.xs + c.row0;
+    o.y = d.y + (int64_t)c.row0 * d.N;
+    o.M = c.rows;
+    o.tile_begin = tiles;
+    tiles += c.tiles;
+  }
+  while (x < kXcds) t.xcd_begin[++x] = tiles;
+  t.total_tiles = tiles;
+  for (int i = 0; i < kXcds; ++i)
+    if (t.xcd_begin[i + 1] - t.xcd_begin[i] > longest) longest = t.xcd_begin[i + 1] - t.xcd_begin[i];
+  grouped_tiled_kernel<256, 256><<<longest * kXcds, 256, 0, s>>>(t);
   return hipGetLastError();
 }
 

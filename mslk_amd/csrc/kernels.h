@@ -90,7 +90,9 @@ struct GroupTable {
   GroupDesc g[kMaxGroupsPerLaunch];
   int count;
   int total_tiles;
+  int xcd_begin[9];   // filled by the launcher: XCD x works on tiles [xcd_begin[x], xcd_begin[x + 1])
 };
+// Takes one descriptor per group (tile_begin ascending); re-cuts them into row chunks dealt to the XCDs by estimated cost.
 hipError_t launch_grouped_tiled(const GroupTable& t, hipStream_t s);
 
 // Groups described in device memory (or uniform); see gemm_grouped.hip for the layouts.
