@@ -542,3 +542,26 @@ def test_quantize_fused_graph_capture():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(y, eager)
+
+
+@pytest.mark.parametrize("N,K", [(8, 1 << 25), (4, 1 << 26)])
+def test_rows_longer_than_the_streaming_kernels_32_bit_offsets(N, K):
+    """The weight-streaming kernel forms 32-bit byte offsets of up to 63 * K + k: K = 2^25 is the last power of two it
+    may take, K = 2^26 has to go to a kernel with 64-bit addressing.  Either way every weight row must be read where it
+    lies (rows differ, so a wrapped offset would show)."""
+    g = torch.Generator(device=DEV).manual_seed(N + (K >> 20))
+    def codes(*shape):
+        mag = torch.randint(0x20, 0x48, shape, dtype=torch.uint8, device=DEV, generator=g)     # |value| in [0.125, 4)
+        sign = torch.randint(0, 2, shape, dtype=torch.uint8, device=DEV, generator=g) << 7
+        return (mag | sign).view(F8)
+    xq, wq = codes(1, K), codes(N, K)
+    xs = torch.full((1,), 2.0 ** -8, device=DEV)
+    ws = torch.rand(N, device=DEV, generator=g) * 1e-3 + 1e-3
+    y = torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xs, ws)
+    torch.cuda.synchronize()
+    ref = torch.zeros(N, dtype=torch.float64, device=DEV)
+    step = 1 << 22
+    for k0 in range(0, K, step):
+        ref += (wq[:, k0:k0 + step].float() * xq[:, k0:k0 + step].float()).double().sum(dim=1)
+    ref = (ref * ws.double() * xs.double()).float().view(1, N)
+    assert_gemm_close(y.cpu(), ref.cpu(), f"N={N} K={K}")
