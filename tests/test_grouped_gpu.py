@@ -34,6 +34,8 @@ def _dev(ts):
     ([64], 512, 512), ([300, 0, 17, 256, 1], 768, 512), ([0, 0, 5], 512, 1024),
     ([128] * 16, 1024, 512), ([7, 300, 0, 0, 513, 64, 2, 1000], 520, 656),
     ([3] * 70, 512, 512),   # more groups than one launch carries in its argument block
+    ([2100, 0, 5, 1030, 256, 257], 768, 512),   # groups cut into panels of four row tiles: row offsets inside a group
+    ([1100] * 40, 512, 512),   # more panels than descriptors: the launch deals whole groups instead
 ])
 def test_tensorlist_grouped(ms, N, K):
     g = torch.Generator().manual_seed(sum(ms) + N + K)
