@@ -59,6 +59,14 @@ __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p
   const void* bias = nullptr;
   if constexpr (BIAS == 1) bias = reinterpret_cast<const float*>(p.bias) + n0;
   if constexpr (BIAS == 2) bias = reinterpret_cast<const uint16_t*>(p.bias) + n0;
+  if constexpr (BIAS == 0 && TS::RING == 0 && TS::NW == 4 && TS::FM * TS::FN * 4 >= 256) {
+    // tiles with every row and column: the epilogue starts inside the last K step
+    if (GemmTile<TS, BIAS, PS>::interior_ok(p.ws + n0, bias, p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K)) {
+      tile.run_interior(lds, p.xq + (int64_t)m0 * p.K, p.wq + (int64_t)n0 * p.K, p.xs + m0, p.ws + n0, bias,
+                        p.y + (int64_t)m0 * p.N + n0, p.N, p.K);
+      return;
+    }
+  }
   tile.run(lds, p.xq + (int64_t)m0 * p.K, p.wq + (int64_t)n0 * p.K, p.xs + m0, p.ws + n0, bias,
            p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K);
 }

@@ -384,6 +384,33 @@ struct GemmTile {
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
   }
 
+  // Whether run_interior() may take the tile: every row and column valid, 16-byte aligned rows of Y and scale / bias
+  // vectors, K a positive multiple of the K step.
+  MSLK_AMD_DEVINL static bool interior_ok(const float* ws, const void* bias, const uint16_t* y, int m_rem, int n_rem, int N, int K) {
+    // (without bias: its 32 values per lane on top of both operands of the step do not fit the registers)
+    return BIAS == 0 && TS::RING == 0 && TS::FM * TS::FN * 4 >= 256 && m_rem >= TS::kBM && n_rem >= TS::kBN && K >= kBK && K % kBK == 0 &&
+           (N & 7) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0 && (reinterpret_cast<uintptr_t>(ws) & 15) == 0 &&
+           (BIAS == 0 || (reinterpret_cast<uintptr_t>(bias) & (BIAS == 1 ? 15 : 7)) == 0);
+  }
+  // run() for such a tile: the epilogue starts inside the last K step.  That step issues no loads, and once the eight
+  // MFMAs of a fragment row are issued its accumulators are final while the rows after it are still being multiplied;
+  // so the step runs fragment row by fragment row, and the scaling, conversion and transpose of row tm - 1 and the
+  // stores of row tm - 2 are issued between the MFMAs of row tm -- the matrix pipe works under the vector
+  // instructions of the epilogue instead of in front of them.  Same arithmetic, same bits.
+  MSLK_AMD_DEVINL void run_interior(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, const float* xs,
+                                    const float* ws, const void* bias, uint16_t* y, int N, int K) {
+    v4f acc[TS::FN][TS::FM];
+    LastStep last;
+    prologue<false>(lds, xq_tile, wq_tile, TS::kBM, TS::kBN, K, (uint32_t)K);
+    accumulate_issued<false, TS::FM, true>(lds, K, acc, &last);
+    // the transposes go into the two WQ buffers that are dead: waves 0, 1 into the first, waves 2, 3 into the second
+    static_assert(TS::NW == 4 && 2 * EPI_WAVE_BYTES <= TS::B_BYTES, "two transpose buffers per free WQ buffer");
+    const int wave = wave_id();
+    char* buf = (wave >> 1 ? last.b_free1 : last.b_free0) + (wave & 1) * EPI_WAVE_BYTES;
+    if (out_f16) epilogue_impl<true, true, true, false, true>(buf, acc, xs, ws, bias, y, TS::kBM, TS::kBN, N, &last);
+    else epilogue_impl<true, false, true, false, true>(buf, acc, xs, ws, bias, y, TS::kBM, TS::kBN, N, &last);
+  }
+
   // K loop of a tile with m_rem valid rows.
   MSLK_AMD_DEVINL void accumulate_rows(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, int m_rem, int n_rem, int K,
                                        uint32_t ld, v4f (&acc)[TS::FN][TS::FM]) {
@@ -433,9 +460,21 @@ struct GemmTile {
   // K loop after prologue() (or, for the symmetric ring, after init()).  DRAIN: the wave has other memory
   // operations in flight behind the prologue loads (the stores of the previous tile's epilogue), so the first wait
   // is for all of them instead of "all but the youngest WQ loads".
-  template <bool DRAIN, int FMV = TS::FM>
-  MSLK_AMD_DEVINL void accumulate_issued(char* lds, int K, v4f (&acc)[TS::FN][TS::FM]) {
+  // What accumulate_issued<..., HOLD_LAST = true> leaves to the caller: the last full K step (its XQ fragments and WQ
+  // fragment 0 in registers, its WQ tile in `b_cur`) and the two WQ buffers nobody touches any more.
+  struct LastStep {
+    v8i xf[TS::FM];
+    v8i wf0;
+    const char* b_cur;
+    char* b_free0;
+    char* b_free1;
+  };
+  // HOLD_LAST (K a positive multiple of the K step, two-plus-three buffers): the last step is not multiplied and the
+  // final barrier is not passed; `last` describes it (see run_interior()).
+  template <bool DRAIN, int FMV = TS::FM, bool HOLD_LAST = false>
+  MSLK_AMD_DEVINL void accumulate_issued(char* lds, int K, v4f (&acc)[TS::FN][TS::FM], LastStep* last = nullptr) {
     static_assert(FMV == TS::FM || TS::RING == 0, "row skipping is built for the two-plus-three buffer tiles");
+    static_assert(!HOLD_LAST || (TS::RING == 0 && FMV == TS::FM), "the held last step belongs to full two-plus-three buffer tiles");
 #pragma unroll
     for (int tn = 0; tn < TS::FN; ++tn)
 #pragma unroll
@@ -466,6 +505,15 @@ struct GemmTile {
           step<true, false, true, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
+        }
+        if constexpr (HOLD_LAST) {
+#pragma unroll
+          for (int tm = 0; tm < TS::FM; ++tm) last->xf[tm] = xf[tm];
+          last->wf0 = wf0;
+          last->b_cur = b_cur;
+          last->b_free0 = b_nxt;
+          last->b_free1 = b_far;
+          return;
         }
         step<false, false, false, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
       }
@@ -566,9 +614,12 @@ struct GemmTile {
   // FULL: every column of the tile is valid and rows of Y are 16-byte aligned; rows may still be ragged unless
   // ALL_ROWS says that the tile has all its rows too.
   // ILV: the m fragments of the tile were dealt to the wave rows round-robin (ragged tiles of the grouped kernels).
-  template <bool FULL, bool F16, bool ALL_ROWS, bool ILV = false>
+  // FUSED: `last` holds the last K step, still to be multiplied; it is multiplied here, fragment row by fragment row,
+  // with the epilogue of the rows that are final issued between its MFMAs (run_interior()).
+  template <bool FULL, bool F16, bool ALL_ROWS, bool ILV = false, bool FUSED = false>
   MSLK_AMD_DEVINL void epilogue_impl(char* buf, v4f (&acc)[TS::FN][TS::FM], const float* xs, const float* ws,
-                                     const void* bias, uint16_t* y, int m_rem, int n_rem, int N) {
+                                     const void* bias, uint16_t* y, int m_rem, int n_rem, int N, LastStep* last = nullptr) {
+    static_assert(!FUSED || (FULL && ALL_ROWS && !ILV && TS::RING == 0), "the fused last step is for interior tiles");
     constexpr int WN = TS::kBN / TS::WN;         // columns per wave
     constexpr int PITCH = WN * 2 + 16;           // bytes per staged row
     constexpr int BUF = 16 * PITCH;
@@ -630,7 +681,8 @@ struct GemmTile {
     const uint32_t lane_off = ((uint32_t)rd_row * (uint32_t)N + (uint32_t)(n_base + rd_chunk * 8)) * 2u;   // bytes; 16 N < 2^31
     constexpr int NP = 16 / RPI;                 // store instructions per 16-row fragment
     constexpr bool ACC_IN_AGPRS = TS::FM * TS::FN * 4 >= 256;
-    if constexpr (ACC_IN_AGPRS) {
+    static_assert(!FUSED || ACC_IN_AGPRS, "the fused last step reads accumulator registers");
+    if constexpr (ACC_IN_AGPRS && !FUSED) {
       // The reads below are opaque to the compiler's hazard handling: 48 wait states let the last MFMA of the K loop
       // (32 cycles) retire before its result is read.
       asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15");
@@ -659,7 +711,7 @@ struct GemmTile {
           // the register allocator moves part of it to vector registers ahead of time, runs out of them and spills,
           // and a reload between the stores waits for all of them.  (Smaller tiles live in vector registers.)
           float a;
-          if constexpr (ACC_IN_AGPRS) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[tn][tm][r]));   // volatile: stays behind the s_nop
+          if constexpr (ACC_IN_AGPRS && !FUSED) asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(a) : "a"(acc[tn][tm][r]));   // volatile: stays behind the s_nop
           else a = acc[tn][tm][r];
           v[r] = (a * wsv[tn][r]) * xsv;   // w_scale first, then x_scale: the order of the reference's epilogue (fp8_rowwise_common.h:66)
           if constexpr (BIAS != 0) v[r] += bv[tn][r];
@@ -683,7 +735,47 @@ struct GemmTile {
       return reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(y + (int64_t)(frag_row(tm) + pass * RPI) * N) + lane_off);
     };
 
-    if constexpr (FULL) {
+    if constexpr (FUSED) {
+      static_assert(TS::FN % NP == 0, "whole n fragments per store");
+      constexpr int TPP = TS::FN / NP;   // n fragments (and MFMAs of a fragment row) per store instruction
+      const FragOff fo = frag_off();
+      const char* b_tile = b_tile_of(last->b_cur);
+      v8i wf[TS::FN];
+      wf[0] = last->wf0;
+#pragma unroll
+      for (int tn = 1; tn < TS::FN; ++tn) wf[tn] = load_frag_b(b_tile, tn, fo);
+      uint4 val[NP];
+      char* dst = reinterpret_cast<char*>(y + (int64_t)frag_row(0) * N) + lane_off;
+      const int64_t dst_step = (int64_t)RPI * N * 2;
+      float xsv = 0.f;
+      __builtin_amdgcn_sched_barrier(0);
+      // iteration t: MFMAs of fragment row t, park of row t - 1 (its MFMAs were issued a whole row, 8 x 32 cycles, ago),
+      // stores of row t - 2
+#pragma unroll
+      for (int t = 0; t < TS::FM + 2; ++t) {
+        if (t >= 2) fetch(t - 2, val);
+        if (t >= 1 && t - 1 < TS::FM) xsv = xs_lds[(t - 1) * 16 + j];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int pass = 0; pass < NP; ++pass) {
+          if (t < TS::FM) {
+#pragma unroll
+            for (int tn = pass * TPP; tn < (pass + 1) * TPP; ++tn)
+              acc[tn][t] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf[tn], last->xf[t], acc[tn][t], 0, 0, 0, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          if (t >= 1 && t - 1 < TS::FM) {
+            park(t - 1, pass * TPP, (pass + 1) * TPP, xsv);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if (t >= 2) {
+            store16_stream(reinterpret_cast<uint16_t*>(dst), val[pass]);
+            dst += dst_step;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+    } else if constexpr (FULL) {
       // With one wave per SIMD nothing else hides the LDS round trip between parking a fragment row and
       // storing it, so the rows are pipelined by hand: the read-back of row tm - 1 is issued before the
       // arithmetic of row tm and its stores follow that arithmetic.
