@@ -74,6 +74,24 @@ def test_exact_when_fp32_accumulation_is_exact(M, N, K):
     assert torch.equal(y.cpu()[:5, :7].double(), small.bfloat16().double())
 
 
+@pytest.mark.parametrize("fp16_out", [False, True])
+@pytest.mark.parametrize("M,N,K", [(3072, 3328, 384), (4096, 4096, 128), (3072, 3072, 256), (3100, 3330, 640)])
+def test_exact_on_full_256_tiles_without_bias(M, N, K, fp16_out):
+    """129 ... 256 tiles of 256 x 256 and no bias: interior tiles run their last K step under the epilogue (K = 128 is
+    that step alone); the last shape adds ragged edge tiles, which take the ordinary epilogue, around them.  Exact
+    arithmetic as above, so every output must match bit for bit."""
+    g = torch.Generator().manual_seed(M + K)
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    xs = 2.0 ** torch.randint(-3, 4, (M,), generator=g).float()
+    ws = 2.0 ** torch.randint(-3, 4, (N,), generator=g).float()
+    want = (xi @ wi.T) * xs[:, None] * ws[None, :]
+    op = torch.ops.mslk.f8f8f16_rowwise if fp16_out else torch.ops.mslk.f8f8bf16_rowwise
+    y = op(*_gpu(xi.to(F8), wi.to(F8), xs, ws))
+    torch.cuda.synchronize()
+    assert torch.equal(y.cpu(), want.half() if fp16_out else want.bfloat16())
+
+
 def test_identity_and_one_hot_weights_select_dequantized_activations():
     g = torch.Generator().manual_seed(9)
     M, K = 300, 512
