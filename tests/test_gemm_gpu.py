@@ -75,10 +75,11 @@ def test_exact_when_fp32_accumulation_is_exact(M, N, K):
 
 
 @pytest.mark.parametrize("fp16_out", [False, True])
+@pytest.mark.parametrize("bias_dtype", [None, torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("M,N,K", [(3072, 3328, 384), (4096, 4096, 128), (3072, 3072, 256), (3100, 3330, 640)])
-def test_exact_on_full_256_tiles_without_bias(M, N, K, fp16_out):
-    """129 ... 256 tiles of 256 x 256 and no bias: interior tiles run their last K step under the epilogue (K = 128 is
-    that step alone); the last shape adds ragged edge tiles, which take the ordinary epilogue, around them.  Exact
+def test_exact_on_full_256_tiles(M, N, K, bias_dtype, fp16_out):
+    """129 ... 256 tiles of 256 x 256: without a bias, interior tiles run their last K step under the epilogue (K = 128
+    is that step alone); the last shape adds ragged edge tiles, which take the ordinary epilogue, around them.  Exact
     arithmetic as above, so every output must match bit for bit."""
     g = torch.Generator().manual_seed(M + K)
     xi = torch.randint(-8, 9, (M, K), generator=g).float()
@@ -86,8 +87,13 @@ def test_exact_on_full_256_tiles_without_bias(M, N, K, fp16_out):
     xs = 2.0 ** torch.randint(-3, 4, (M,), generator=g).float()
     ws = 2.0 ** torch.randint(-3, 4, (N,), generator=g).float()
     want = (xi @ wi.T) * xs[:, None] * ws[None, :]
+    bias = None
+    if bias_dtype is not None:
+        bias = torch.randint(-4, 5, (N,), generator=g).float()
+        want = want + bias[None, :]
+        bias = bias.to(bias_dtype).to(DEV)
     op = torch.ops.mslk.f8f8f16_rowwise if fp16_out else torch.ops.mslk.f8f8bf16_rowwise
-    y = op(*_gpu(xi.to(F8), wi.to(F8), xs, ws))
+    y = op(*_gpu(xi.to(F8), wi.to(F8), xs, ws), bias=bias)
     torch.cuda.synchronize()
     assert torch.equal(y.cpu(), want.half() if fp16_out else want.bfloat16())
 
