@@ -253,6 +253,65 @@ def _vendor_sweep(api):
                       "min_ratio": round(ratios[0], 3), "max_ratio": round(ratios[-1], 3)}))
 
 
+def _ceilings(api):
+    """`--only ceilings`: what this GPU sustains on the two resources the roofline fractions are priced against, from
+    kernels that live in the library (mslk_amd_debug_stream_read / mslk_amd_debug_mfma_loop): a pure read of HBM-resident
+    buffers (register loads and the LDS-DMA loads of the GEMM kernels, the decode weight size and 1 GiB) and a
+    register-only FP8 MFMA loop in both instruction forms on zeros, uniform random codes and the codes of the cfg1
+    operands.  Prints one JSON line."""
+    import torch
+    import mslk_amd
+    from mslk_amd import workloads as W
+    dev = "cuda:0"
+    L = api.L
+    out = {}
+    sink = torch.zeros(16, dtype=torch.int32, device=dev)
+    # ---- streaming read: six distinct 64 MiB buffers (more than the 256 MB Infinity Cache) and one 1 GiB buffer
+    small = [torch.randint(0, 255, (64 << 20,), dtype=torch.uint8, device=dev) for _ in range(6)]
+    big = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
+    for mode, mname in ((0, "register_loads"), (1, "lds_dma_loads")):
+        for label, bufs in (("64MiB", small), ("1GiB", [big])):
+            best = None
+            for wgs in (512, 1024, 2048, 4096):
+                def step(i, bufs=bufs, wgs=wgs, mode=mode):
+                    b = bufs[i % len(bufs)]
+                    api.check(L.mslk_amd_debug_stream_read(b.data_ptr(), b.numel(), mode, wgs, sink.data_ptr(), api.stream))
+                _settle(step, 10.0)
+                ms = _median_events_ms(step, 30 if label == "64MiB" else 6)
+                if best is None or ms < best[0]:
+                    best = (ms, wgs)
+            nbytes = bufs[0].numel()
+            out[f"stream_read_{mname}_{label}"] = {"ms": best[0], "workgroups": best[1], "TBps": nbytes / (best[0] * 1e-3) / 1e12,
+                                                   "frac_of_8TBps": nbytes / (best[0] * 1e-3) / PEAK_HBM_BPS}
+    del small, big
+    # the launch itself: the same kernel on 16 bytes
+    tiny = torch.zeros(1024, dtype=torch.uint8, device=dev)
+    out["empty_launch_us"] = _median_events_ms(
+        lambda i: api.check(L.mslk_amd_debug_stream_read(tiny.data_ptr(), 1024, 0, 256, sink.data_ptr(), api.stream)), 200) * 1e3
+    # ---- register-only MFMA loops: 256 workgroups x 4 waves x iters x 2 * 128^3 FLOP
+    wl = W.cfg1()
+    xq, _ = mslk_amd.quantize_fp8_row(wl.x[:64].to(dev), use_triton=False)
+    wq, _ = mslk_amd.quantize_fp8_row(wl.w[:64].to(dev), use_triton=False)
+    cfg1_codes = torch.cat([xq.view(torch.uint8).reshape(-1)[:65536], wq.view(torch.uint8).reshape(-1)[:65536]]).contiguous()
+    rnd = torch.randint(0, 255, (131072,), dtype=torch.uint8, device=dev)
+    rnd[(rnd & 0x7F) == 0x7F] = 0x30                      # no NaN codes
+    datas = (("zeros", torch.zeros(131072, dtype=torch.uint8, device=dev)), ("uniform_random_codes", rnd),
+             ("cfg1_operand_codes", cfg1_codes))
+    iters, wgs = 512, 256
+    flops = wgs * 4 * iters * 2.0 * 128 ** 3
+    fsink = torch.zeros(16, device=dev)
+    for dname, data in datas:
+        for form, fname in ((0, "16x16x128"), (1, "32x32x64")):
+            def step(i, data=data, form=form):
+                api.check(L.mslk_amd_debug_mfma_loop(data.data_ptr(), form, iters, wgs, fsink.data_ptr(), api.stream))
+            _settle(step, 30.0)
+            ms = _median_events_ms(step, 20)
+            out[f"mfma_loop_{fname}_{dname}"] = {"ms": ms, "PFLOPs": flops / (ms * 1e-3) / 1e15,
+                                                 "frac_of_5PF": flops / (ms * 1e-3) / PEAK_FP8_FLOPS,
+                                                 "implied_clock_GHz": flops / (ms * 1e-3) / (256 * 4 * 2048.0) / 1e9}
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -261,7 +320,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", default="",
-                    help="helper: run only this piece (gemm|gemm-timed|quantize|decode|cfg2|grouped|traffic|vendor) and exit")
+                    help="helper: run only this piece (gemm|gemm-timed|quantize|decode|cfg2|grouped|traffic|vendor|ceilings) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -278,6 +337,9 @@ def main():
     extras = {}
     if args.only == "vendor":
         _vendor_sweep(api)
+        return
+    if args.only == "ceilings":
+        _ceilings(api)
         return
 
     # ---------------------------------------------------------------- cfg1: 4096^3

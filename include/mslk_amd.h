@@ -289,6 +289,20 @@ int mslk_amd_f8f8bf16_rowwise_batched(const void* xq, const void* wq, const floa
  */
 int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stream);
 
+/*
+ * Ceiling probes for the benchmark's roofline columns; no counterpart in the reference (its bench divides by fixed
+ * peak figures, bench/gemm/gemm_bench.py:61-68) and not part of the product path.
+ *   mslk_amd_debug_stream_read: `workgroups` x 256 lanes read `bytes` from `src` once and write nothing.  mode 0: 16-byte
+ *     non-temporal loads into registers (bytes % 16 == 0); mode 1: the global -> LDS DMA loads the GEMM kernels use
+ *     (bytes % 1024 == 0).  `sink` (device int, may be NULL) is never written for real inputs.
+ *   mslk_amd_debug_mfma_loop: `workgroups` x 4 waves each run `iters` iterations of a 128 x 128 x 128 wave tile out of
+ *     registers: 64 v_mfma_f32_16x16x128_f8f6f4 (form 0) or 32 v_mfma_f32_32x32x64_f8f6f4 (form 1) per iteration, i.e.
+ *     iters * 2 * 128^3 FLOP per wave.  `operands` points at 128 KiB of e4m3 codes (32-byte aligned) that fill the operand
+ *     registers once; the rate depends on these values through the power they draw.
+ */
+int mslk_amd_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, void* stream);
+int mslk_amd_debug_mfma_loop(const void* operands, int form, int iters, int workgroups, void* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -419,4 +419,21 @@ int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stre
   return check_hip(launch_cast_e4m3fn(in, n, out, (hipStream_t)stream), "cast launch");
 }
 
+int mslk_amd_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, void* stream) {
+  if (mode != 0 && mode != 1) return fail("debug_stream_read: mode must be 0 (register loads) or 1 (LDS DMA loads)");
+  if (bytes < 0 || bytes % (mode == 0 ? 16 : 1024) != 0) return fail("debug_stream_read: bytes must be a non-negative multiple of %d", mode == 0 ? 16 : 1024);
+  if (workgroups <= 0 || workgroups > 65536) return fail("debug_stream_read: workgroups must be in 1 .. 65536");
+  if (bytes == 0) return 0;
+  if (!src || reinterpret_cast<uintptr_t>(src) % 16 != 0) return fail("debug_stream_read: src must be a 16-byte aligned device pointer");
+  return check_hip(launch_debug_stream_read(src, bytes, mode, workgroups, sink, (hipStream_t)stream), "stream read launch");
+}
+
+int mslk_amd_debug_mfma_loop(const void* operands, int form, int iters, int workgroups, void* sink, void* stream) {
+  if (form != 0 && form != 1) return fail("debug_mfma_loop: form must be 0 (16x16x128) or 1 (32x32x64)");
+  if (iters < 0 || iters > (1 << 20)) return fail("debug_mfma_loop: iters must be in 0 .. 2^20");
+  if (workgroups <= 0 || workgroups > 65536) return fail("debug_mfma_loop: workgroups must be in 1 .. 65536");
+  if (!operands || reinterpret_cast<uintptr_t>(operands) % 32 != 0) return fail("debug_mfma_loop: operands must be a 32-byte aligned device pointer to 128 KiB");
+  return check_hip(launch_debug_mfma_loop(operands, form, iters, workgroups, sink, (hipStream_t)stream), "mfma loop launch");
+}
+
 }  // extern "C"

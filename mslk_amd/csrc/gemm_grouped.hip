@@ -111,7 +111,10 @@ MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
     const int lane = threadIdx.x & 63;
     // Every quantity fits 32 bits (the host checks the dimensions and the grid): sizes beyond the tensor mark the group bad.
     struct Chunk { int start, len, tiles, incl; bool bad; };
-    auto load_chunk = [&](int base, int& carry_len) {
+    // `seen_bad` carries "an earlier group was inconsistent" from chunk to chunk: such a group and every group after it
+    // own no tiles, so the tile count, the XCD slices and the lookup all stop at the first bad group and every tile
+    // of the groups in front of it gets a workgroup (the grid is sized for consistent extents).
+    auto load_chunk = [&](int base, int& carry_len, bool& seen_bad) {
       Chunk c;
       const int gi = base + lane;
       const bool in = gi < p.G;
@@ -148,7 +151,10 @@ MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
           c.len = c.bad ? 0 : (int)len64;
         }
       }
-      c.tiles = (in && !c.bad) ? ((c.len + blk - 1) / blk) * fixed_tiles : 0;
+      const unsigned long long bad_lanes = __ballot(c.bad);
+      const bool after_bad = seen_bad || (bad_lanes != 0 && lane >= __ffsll((long long)bad_lanes) - 1);
+      seen_bad = seen_bad || bad_lanes != 0;
+      c.tiles = (in && !after_bad) ? ((c.len + blk - 1) / blk) * fixed_tiles : 0;
       c.incl = c.tiles;
 #pragma unroll
       for (int d = 1; d < 64; d <<= 1) {
@@ -159,19 +165,22 @@ MSLK_AMD_DEVINL bool find_group(const DeviceGroups& p, int t, GroupSpan& sp) {
     };
     int64_t total_tiles = 0;
     int carry_len = 0;
-    Chunk first = load_chunk(0, carry_len);
+    bool seen_bad = false;
+    Chunk first = load_chunk(0, carry_len, seen_bad);
+    const bool first_bad = seen_bad;
     total_tiles = __shfl(first.incl, 63, 64);
-    for (int base = 64; base < p.G; base += 64) total_tiles += __shfl(load_chunk(base, carry_len).incl, 63, 64);
+    for (int base = 64; base < p.G && !seen_bad; base += 64) total_tiles += __shfl(load_chunk(base, carry_len, seen_bad).incl, 63, 64);
     const int64_t per_xcd = (total_tiles + kXcds - 1) / kXcds;
     const int64_t slot = t / kXcds;                       // `t` arrives as the workgroup id
     const int64_t tile = (int64_t)(t % kXcds) * per_xcd + slot;
     if (slot >= per_xcd || tile >= total_tiles) return false;
     int64_t carry_tiles = 0;
     carry_len = 0;
+    seen_bad = first_bad;
     for (int base = 0; base < p.G; base += 64) {
       Chunk c = first;
       if (base == 0) carry_len = __shfl(first.start + first.len, 63, 64);   // sizes: rows of the first 64 groups
-      else c = load_chunk(base, carry_len);
+      else c = load_chunk(base, carry_len, seen_bad);
       const int64_t excl = carry_tiles + c.incl - c.tiles;
       const bool hit = c.tiles > 0 && tile >= excl && tile < excl + c.tiles;
       const unsigned long long hit_mask = __ballot(hit), bad_mask = __ballot(c.bad);

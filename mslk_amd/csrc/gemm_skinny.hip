@@ -388,8 +388,9 @@ hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
 //      wave, wave + 8, ...: next to their weight loads it fetches the bf16 activations of just these steps (M * 256 bytes
 //      per step, 8 elements per lane and load), converts them in registers and parks the codes in its private LDS
 //      buffer, from where the MFMA fragment is two 16-byte reads.  The conversion work of a workgroup is therefore M * K
-//      elements split over its 512 lanes.  No scale_ub here, so no product exceeds 448 (1 + 2^-22) and the conversion
-//      needs no overflow fix-up; NaN stays NaN.
+//      elements split over its 512 lanes.  No scale_ub here, so in a row with a finite maximum no product exceeds
+//      448 (1 + 2^-22) and the conversion needs no overflow fix-up; rows with a NaN or an infinity take the quantizer's
+//      own conversion routine.
 // Workgroup 0 also writes the codes and the scales out when the caller wants them.
 // ---------------------------------------------------------------------------------------------
 MSLK_AMD_DEVINL v2i quantize8_bf16(v4i raw, float inv) {
@@ -404,6 +405,13 @@ MSLK_AMD_DEVINL v2i quantize8_bf16(v4i raw, float inv) {
   lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
   int hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false);
   hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+  // A row whose maximum is NaN or infinite has inv = NaN or 0 and NaN products (NaN * x, inf * 0); only such a row can
+  // hold anything the plain conversion does not settle.  It takes the stand-alone quantizer's conversion, which forces
+  // sign | 0x7F, so that the codes written out are that kernel's bits for every input, NaN signs included.
+  if (!(inv > 0.f && inv < __builtin_inff())) {
+    lo = (int)(cvt_pk_e4m3fn(f[0], f[1]) | (cvt_pk_e4m3fn(f[2], f[3]) << 16));
+    hi = (int)(cvt_pk_e4m3fn(f[4], f[5]) | (cvt_pk_e4m3fn(f[6], f[7]) << 16));
+  }
   return v2i{lo, hi};
 }
 

@@ -80,8 +80,29 @@ MSLK_AMD_DEVINL void store16_stream(uint16_t* dst, uint4 val) {
   asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
 }
 
-MSLK_AMD_DEVINL void dma16(const uint8_t* g, char* lds_wave_base) {
-  __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_wave_base, 16, 0, 0);
+// Global -> LDS copy of 16 bytes per lane (1 KiB per wave, contiguous in LDS from `lds_wave_base`), addressed as
+// wave-uniform base + 32-bit lane offset.  Written as an instruction instead of the compiler's builtin for two reasons:
+//   * while a load the compiler knows of as "writes LDS through the vector memory path" is in flight, every wait it
+//     inserts for an LDS read becomes lgkmcnt(0) -- all reads, not the one whose value is needed.  The K loop always has
+//     loads in flight, and its fragment re-loads (sixteen reads behind the barrier, the first MFMA of the next step needs
+//     the first four) waited for the last of them.  With the load opaque the compiler counts its LDS reads exactly;
+//   * the address stays "scalar base + 32-bit vector offset" (the builtin's address was kept as sixteen 64-bit vector
+//     pairs and advanced by a vector instruction per load).
+// Consequences the callers carry: the compiler sees neither the LDS write nor the outstanding load, so every read of
+// the copied bytes sits behind an explicit s_waitcnt vmcnt (wait_and_barrier / wait_vmcnt0) -- none relies on a wait the
+// compiler would have inserted -- and the "memory" clobber keeps LDS accesses from moving across the statement.  No
+// register receives data, so there is nothing the register allocator could reuse too early.  M0 (the LDS address of
+// the copy) is written inside the statement and declared clobbered; nothing else in these kernels uses M0.  One wait
+// state separates the M0 write from the load.  A violation shows in the bit-exact tests of tests/test_exact_paths_gpu.py
+// and tests/test_gemm_gpu.py::test_exact_on_full_256_tiles (stale or missing operand bytes change integer sums).
+MSLK_AMD_DEVINL const uint8_t* uniform_ptr(const uint8_t* p) {
+  const uint64_t v = reinterpret_cast<uint64_t>(p);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v), hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
+}
+MSLK_AMD_DEVINL void dma16(const uint8_t* base, uint32_t off, char* lds_wave_base) {
+  const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr_t)lds_wave_base;
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(dst) : "memory", "m0");
 }
 
 
@@ -106,8 +127,9 @@ struct GemmTile {
     int lane = threadIdx.x & 63;
     asm volatile("" : "+v"(lane));   // recompute the row / chunk of each load per tile instead of keeping 32 values live
     const int wave = wave_id();
-    a_base = xq_tile;
-    b_base = wq_tile;
+    // the tile pointers are the same in every lane; say so, so that the DMA loads get their base in scalar registers
+    a_base = uniform_ptr(xq_tile);
+    b_base = uniform_ptr(wq_tile);
     a_rows = rows_a;
 #pragma unroll
     for (int i = 0; i < TS::LA; ++i) {
@@ -139,11 +161,11 @@ struct GemmTile {
   // DMA load number i (0 .. LA-1 for the XQ tile, 0 .. LB-1 for the WQ tile) of the K step at byte k0.
   // `abuf` / `bbuf` are the LDS buffers that receive the XQ / WQ tile of the K step at byte k0.
   MSLK_AMD_DEVINL void issue_a(char* abuf, int k0, int i) {
-    dma16(a_base + k0 + a_off[i], abuf + (wave_id() * TS::LA + i) * 1024);
+    dma16(a_base + k0, a_off[i], abuf + (wave_id() * TS::LA + i) * 1024);
   }
   MSLK_AMD_DEVINL void issue_b(char* bbuf, int k0, int i) {
     // pre-shuffled: the K step at byte k0 starts 16 rows x k0 bytes into the row group
-    dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
+    dma16(b_base + (PS ? k0 * 16 : k0), b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
   }
   MSLK_AMD_DEVINL void issue_a_all(char* abuf, int k0) {
 #pragma unroll
@@ -168,7 +190,7 @@ struct GemmTile {
       const int row = (wave * TS::LA + i) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swz(row);
       char* dst = abuf + (wave * TS::LA + i) * 1024;
-      if (chunk * 16 < k_valid) dma16(a_base + k0 + a_off[i], dst);
+      if (chunk * 16 < k_valid) dma16(a_base + k0, a_off[i], dst);
       else *reinterpret_cast<uint4*>(dst + lane * 16) = make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
@@ -177,7 +199,7 @@ struct GemmTile {
       const int chunk = (lane & 7) ^ lds_swz(row);
       char* dst = bbuf + (wave * TS::LB + i) * 1024;
       const bool valid = PS ? ((wave * TS::LB + i) & 1) * 64 < k_valid : chunk * 16 < k_valid;
-      if (valid) dma16(b_base + (PS ? k0 * 16 : k0) + b_off[i], dst);
+      if (valid) dma16(b_base + (PS ? k0 * 16 : k0), b_off[i], dst);
       else *reinterpret_cast<uint4*>(dst + lane * 16) = make_uint4(0, 0, 0, 0);
     }
   }
@@ -271,6 +293,16 @@ struct GemmTile {
       step_rows<DMA_A, DMA_B, NEXT, PENDING, FMV>(b_cur, a_dst, a_nxt, b_nxt, b_far, k_a, k_b, acc, xf, wf0);
       return;
     }
+    v8i wf_last;
+    step_head<DMA_A, DMA_B>(b_cur, a_dst, b_far, k_a, k_b, acc, xf, wf0, wf_last);
+    step_tail<NEXT, PENDING>(a_nxt, b_nxt, acc, xf, wf0, wf_last);
+  }
+
+  // The part of a full-tile K step in front of its barrier: every n fragment but the last, with the step's DMA loads.
+  // Leaves the last WQ fragment of the step in `wf_last`.
+  template <bool DMA_A, bool DMA_B>
+  MSLK_AMD_DEVINL void step_head(const char* b_cur, char* a_dst, char* b_far, int k_a, int k_b, v4f (&acc)[TS::FN][TS::FM],
+                                 v8i (&xf)[TS::FM], const v8i& wf0, v8i& wf_last) {
     constexpr int HALF = TS::FN / 2;
     static_assert((TS::LA + TS::LB) % HALF == 0, "DMA loads spread evenly over the first half");
     constexpr int NDMA = (TS::LA + TS::LB) / HALF;   // DMA loads per MFMA group
@@ -291,6 +323,23 @@ struct GemmTile {
       for (int tm = 0; tm < TS::FM; ++tm) {
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
         if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
+        // Large tiles (at most one load per MFMA): the loads of a step are spread over ALL groups in front of the barrier,
+        // XQ first, so that the load path sees them at an even rate.
+        constexpr int ND = TS::LA + TS::LB, GD = TS::FN - 1;
+        const int first = (tn * ND + GD - 1) / GD, next = ((tn + 1) * ND + GD - 1) / GD;   // group tn issues loads [first, next)
+        const int ds = tm - (TS::FM - (next - first));
+        if (PER_SLOT == 1 && ND <= GD * TS::FM) {
+          if (ds >= 0) {
+            const int q = first + ds;
+            if (q < TS::LA) {
+              if constexpr (DMA_A) issue_a(a_dst, k_a, q);
+            } else {
+              if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
+            }
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          continue;
+        }
         const int d = tm - (TS::FM - SLOTS);
         if (tn < HALF && d >= 0) {
 #pragma unroll
@@ -310,6 +359,15 @@ struct GemmTile {
       wf = wf_next;
       __builtin_amdgcn_sched_barrier(0);
     }
+    wf_last = wf;
+  }
+
+  // The rest of the step: the barrier (NEXT), then the last n fragment, whose XQ fragments are replaced by those of the
+  // next step as they retire.
+  template <bool NEXT, int PENDING>
+  MSLK_AMD_DEVINL void step_tail(const char* a_nxt, const char* b_nxt, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0,
+                                 const v8i& wf_last) {
+    const FragOff fo = frag_off();
     if constexpr (NEXT) {
       wait_and_barrier<PENDING>();
       wf0 = load_frag_b(b_tile_of(b_nxt), 0, fo);
@@ -317,7 +375,7 @@ struct GemmTile {
     const char* a_next = a_tile_of<false>(a_nxt);
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
-      acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+      acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf_last, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
       if constexpr (NEXT) {
         xf[tm] = load_frag_a<false>(a_next, tm, fo);
         __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
@@ -556,6 +614,7 @@ struct GemmTile {
     if (k_tail > 0) {
       __syncthreads();   // everybody is done with the buffers of the full steps before one pair is refilled
       issue_loads_tail(a_tail, b_tail, KT * kBK, k_tail);
+      wait_vmcnt0();    // the DMA loads are not visible to the compiler: the wait is explicit
       __syncthreads();
       load_first_frags<FMV>(a_tail, b_tail, xf, wf0);
       step<false, false, false, 0, FMV>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);

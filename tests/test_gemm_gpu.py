@@ -547,6 +547,30 @@ def test_quantize_fused_into_the_decode_gemm(M, N, K, bias_dtype):
         assert torch.isnan(y[(~finite).to(DEV)].float()).any(dim=1).all()
 
 
+def test_quantize_fused_gives_the_quantizer_bits_for_negative_nan_and_infinity():
+    """The codes and scales the one-launch path writes out are the stand-alone quantizer's for every input: rows with
+    -NaN, -inf, +NaN and +inf elements are compared byte for byte (sign bits of the NaN codes included) with
+    quantize_fp8_row(use_triton=False) on the same device."""
+    g = torch.Generator().manual_seed(5)
+    M, N, K = 4, 520, 2048
+    x = torch.randn(M, K, generator=g).bfloat16()
+    bits = x.view(torch.int16)
+    bits[0, 33] = -64            # 0xFFC0: negative quiet NaN
+    bits[1, 1000] = -128         # 0xFF80: -inf
+    bits[2, 5] = 0x7FC0          # +NaN ...
+    bits[2, 6] = -128            # ... and -inf in the same row
+    x[3, 77] = float("inf")
+    x[3, 78] = -3.0
+    wq, ws = O.quantize_fp8_row((torch.randn(N, K, generator=g) * 0.02).bfloat16())
+    xd = x.to(DEV)
+    y, xq, xs = torch.ops.mslk.quantize_f8f8bf16_rowwise(xd, wq.to(DEV), ws.to(DEV))
+    q2, s2 = mslk_amd.quantize_fp8_row(xd, use_triton=False)
+    torch.cuda.synchronize()
+    assert torch.equal(xq.view(torch.uint8), q2.view(torch.uint8)), "codes differ from the stand-alone quantizer"
+    assert torch.equal(xs.view(torch.int32), s2.view(torch.int32)), "scale bits differ from the stand-alone quantizer"
+    assert (xq.view(torch.uint8)[0] & 0x7F == 0x7F).all() and torch.isnan(xs[0])   # a NaN row is NaN codes throughout
+
+
 def test_quantize_fused_graph_capture():
     g = torch.Generator().manual_seed(77)
     x = torch.randn(4, 4096, generator=g).bfloat16().to(DEV)

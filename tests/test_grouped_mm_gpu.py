@@ -169,6 +169,22 @@ def test_inconsistent_offsets_write_nothing_out_of_range():
     assert (out[64:] == SENTINEL).all()
 
 
+def test_groups_after_an_inconsistent_one_take_no_workgroups_from_the_valid_ones():
+    """Offsets [M, 0, M, 0, M, 0]: group 0 owns every row, group 1 ends before it starts, and the groups after it look
+    valid again.  Every tile of group 0 must be computed (the tile count that cuts the list into XCD slices stops at the
+    first bad group; counting the later ones would leave tiles of group 0 without a workgroup) and nothing else touched."""
+    g = torch.Generator().manual_seed(7)
+    M, N, K, G = 2048, 512, 512, 6
+    xq, xs = _quant(M, K, g)
+    wq, ws = _quant(G * N, K, g, 0.02)
+    out = _sentinel(M, N)
+    ends = torch.tensor([M, 0, M, 0, M, 0], dtype=torch.int32, device=DEV)
+    torch.ops.mslk.f8f8bf16_rowwise_grouped_mm(xq.to(DEV), wq.view(G, N, K).to(DEV), xs.to(DEV), ws.view(G, N).to(DEV), ends, out)
+    torch.cuda.synchronize()
+    assert not (out == SENTINEL).all(dim=1).any(), "rows of the valid first group were left uncomputed"
+    assert_gemm_close(out, O.dequant_matmul(xq, wq[:N], xs, ws[:N]))
+
+
 @pytest.mark.parametrize("sizes", [[64, 10000], [64, 2 ** 40], [64, -3, 20], [64] + [2 ** 30] * 4 + [32], [2 ** 31 - 1, 2 ** 31 - 1, 2]])
 def test_inconsistent_sizes_of_the_stacked_entry_point_write_nothing_out_of_range(sizes):
     """int64 group sizes that do not fit the tensor (too large, negative, or adding up past 2^31 so that a 32-bit running sum
