@@ -29,10 +29,13 @@ PEAK_FP8_FLOPS_REF = 4.6e15  # the figure the reference's bench uses for gfx950 
 PEAK_HBM_BPS = 8.0e12
 
 
+TRAFFIC_SOURCE = "profiles/gemm_4096_traffic_pmc.txt"
+
+
 def _measured_traffic_bytes():
     """HBM-side bytes per 4096^3 GEMM launch from the committed rocprofv3 FETCH_SIZE/WRITE_SIZE summary
     (counters cannot be read from inside this process); None when the summary is absent."""
-    path = os.path.join(ROOT, "profiles", "gemm_4096_traffic_pmc.txt")
+    path = os.path.join(ROOT, *TRAFFIC_SOURCE.split("/"))
     try:
         for ln in open(path):
             if ln.startswith("traffic per launch ="):
@@ -320,7 +323,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", default="",
-                    help="helper: run only this piece (gemm|gemm-timed|quantize|decode|cfg2|grouped|traffic|vendor|ceilings) and exit")
+                    help="helper: run only this piece (gemm|gemm-timed|power|quantize|decode|cfg2|grouped|traffic|vendor|ceilings) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -371,7 +374,7 @@ def main():
         print(json.dumps({"copy_bytes_each_way": 256 << 20, "gemm_launches": 12}))
         return
     settle_launches = 0
-    if args.only in ("", "gemm", "gemm-timed"):
+    if args.only in ("", "gemm", "gemm-timed", "power"):
         settle_launches = _settle(gemm_step)      # outside the timed region, named in config.workload
         for i in range(args.warmup):
             gemm_step(i)
@@ -396,6 +399,29 @@ def main():
         extras["gemm_cfg1_graph_replay"] = {"ms": graph_ms, "TFLOPs": flops / (graph_ms * 1e-3) / 1e12,
                                             "frac_mfma": flops / (graph_ms * 1e-3) / PEAK_FP8_FLOPS,
                                             "note": "120 launches in one HIP graph, same operand rotation"}
+        if (not args.no_extras and args.only == "") or args.only == "power":
+            # The same launches on all-zero codes: the matrix cores then draw little power and the clock stays at its
+            # maximum, so the difference to the timed run is what the power limit costs on this data (the schedule, the
+            # bytes moved and the instruction stream are identical).  Not a performance claim.
+            zsets = [(torch.zeros_like(xq0), torch.zeros_like(wq0), xs0, ws0, sets[j][4]) for j in range(NSETS)]
+
+            def zero_step(i):
+                xq, wq, xs, ws, y = zsets[i % NSETS]
+                api.gemm(xq, wq, xs, ws, y)
+
+            _settle(zero_step)
+            z_ms = _median_events_ms(zero_step, 200)
+            _settle(gemm_step)
+            r_ms = _median_events_ms(gemm_step, 200)
+            extras["gemm_cfg1_zero_operands"] = {"ms": z_ms, "TFLOPs": flops / (z_ms * 1e-3) / 1e12,
+                                                 "frac_mfma": flops / (z_ms * 1e-3) / PEAK_FP8_FLOPS,
+                                                 "ms_real_operands_same_loop": r_ms,
+                                                 "note": "same kernel, same bytes, all-zero codes: what the launch costs when the "
+                                                         "power limit does not bind (see bench.py --only ceilings)"}
+            del zsets
+            if args.only == "power":
+                print(json.dumps(extras))
+                return
         if not args.no_extras and args.only == "":
             # For scale only: the vendor library (hipBLASLt behind torch._scaled_mm, row-wise scales) on the same
             # operand rotation.  Not part of the product path and not a fallback.
@@ -563,6 +589,13 @@ def main():
                                 "GBps_graph_replay": nbytes / (ms_graph * 1e-3) / 1e9,
                                 "ms_preshuffled_weights": ms_ps, "GBps_preshuffled_weights": nbytes / (ms_ps * 1e-3) / 1e9,
                                 "frac_hbm_preshuffled_weights": nbytes / (ms_ps * 1e-3) / PEAK_HBM_BPS, **fused, "parity": par}
+        for k, d in decode.items():
+            # what a deployer gets per M after offline weight preparation: the faster of the row-major and the
+            # pre-shuffled weight layout (both are operators of the path; the weights are re-laid out once, offline)
+            best = min(d["ms"], d["ms_preshuffled_weights"])
+            d["best_layout"] = "preshuffled" if d["ms_preshuffled_weights"] < d["ms"] else "row-major"
+            d["ms_best_layout"] = best
+            d["frac_hbm_best_layout"] = d["bytes"] / (best * 1e-3) / PEAK_HBM_BPS
         extras["decode_N8192_K8192"] = decode
         del wsets, wshuf
         if args.only == "decode":
@@ -575,6 +608,7 @@ def main():
         a, sa = mslk_amd.quantize_fp8_row(wl0.x.to(dev), use_triton=False)
         b, sb = mslk_amd.quantize_fp8_row(wl0.w.to(dev), use_triton=False)
         y0 = torch.empty(1024, 1024, dtype=torch.bfloat16, device=dev)
+        _settle(lambda i: api.gemm(a, b, sa, sb, y0), 20.0)
         ms = _median_events_ms(lambda i: api.gemm(a, b, sa, sb, y0), 100)
         extras["gemm_cfg0_1024"] = {"ms": ms, "TFLOPs": 2.0 * 1024**3 / (ms * 1e-3) / 1e12, "parity": _parity(y0, a, b, sa, sb)}
 
@@ -611,9 +645,17 @@ def main():
         _settle(lambda i: call4())   # the first few dozen launches on freshly allocated 640 MiB of weights run up to 25 % slower
         ms = _median_events_ms(lambda i: call4(), 10)
         f4 = 2.0 * 8192 * 8192 * 5120
+        # the same call through the operator (argument checks, output allocation and marshalling of 80 pointers in Python)
+        ms_op = _median_events_ms(lambda i: torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4), 10)
+        t0 = time.perf_counter()
+        for _ in range(20):
+            torch.ops.mslk.f8f8bf16_rowwise_grouped(xl, wq4, sl, ws4)
+        host_us = (time.perf_counter() - t0) / 20 * 1e6   # launches are asynchronous: this is host time per call
+        torch.cuda.synchronize()
         par4 = [_parity(ys4[e], xl[e], wq4[e], sl[e], ws4[e]) for e in range(16) if wl4.counts[e]]
         extras["grouped_cfg4_16x8192x5120"] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12,
                                                 "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS, "counts": wl4.counts,
+                                                "ms_through_torch_ops": ms_op, "host_us_per_torch_ops_call": host_us,
                                                 "parity": {"max_rel": max(p["max_rel"] for p in par4),
                                                            "normwise": max(p["normwise"] for p in par4),
                                                            "elementwise_violations": sum(p["elementwise_violations"] for p in par4),
@@ -639,8 +681,14 @@ def main():
             api.check(L.mslk_amd_f8f8bf16_rowwise_batched(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
                                                           None, 0, 16, 512, 8192, 5120, y4.data_ptr(), api.stream))
 
+        one = torch.tensor([8192], dtype=torch.int64, device=dev)
+
+        def single_group_call():   # one expert takes all 8192 rows: its 40 MiB of weights stay in the Infinity Cache
+            api.check(L.mslk_amd_f8f8bf16_rowwise_grouped_stacked(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
+                                                                  one.data_ptr(), 1, 8192, 8192, 5120, y4.data_ptr(), api.stream))
+
         for name, call in (("grouped_stacked_cfg4", stacked_call), ("grouped_mm_2d3d_cfg4", offsets_call),
-                           ("batched_16x512x8192x5120", batched_call)):
+                           ("batched_16x512x8192x5120", batched_call), ("grouped_one_warm_group_8192x8192x5120", single_group_call)):
             _settle(lambda i: call(), 20.0)
             ms = _median_events_ms(lambda i: call(), 10)
             extras[name] = {"ms": ms, "TFLOPs": f4 / (ms * 1e-3) / 1e12, "frac_mfma": f4 / (ms * 1e-3) / PEAK_FP8_FLOPS}
@@ -668,7 +716,9 @@ def main():
         "pct_of_reference_peak_4.6PF": 100.0 * value * 1e12 / PEAK_FP8_FLOPS_REF,
         "roofline": {"kernel": "dense_tiled_kernel<256,256> (f8f8bf16_rowwise 4096^3)", "bound": "mfma",
                      "achieved": achieved, "peak": PEAK_FP8_FLOPS / 1e12, "unit": "TFLOP/s",
-                     "frac": achieved * 1e12 / PEAK_FP8_FLOPS, "traffic": _measured_traffic_bytes(), "kernel_ms": kern_ms,
+                     "frac": achieved * 1e12 / PEAK_FP8_FLOPS, "traffic": _measured_traffic_bytes(),
+                     "traffic_source": f"{TRAFFIC_SOURCE} (rocprofv3 counters of an earlier run of this command, not measured in this run)",
+                     "kernel_ms": kern_ms,
                      "flops_per_launch": flops},
         "cpu_baseline": cpu,
         "extras": extras,

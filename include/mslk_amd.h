@@ -290,6 +290,19 @@ int mslk_amd_f8f8bf16_rowwise_batched(const void* xq, const void* wq, const floa
 int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stream);
 
 /*
+ * Which kernel the dense entry points (mslk_amd_f8f8bf16_rowwise, mslk_amd_f8f8f16_rowwise, mslk_amd_f8f8_rowwise_preshuffle)
+ * pick for a shape, as text ("dense_tiled<256,256,waves=2x2,ring=0> tiles=256", "skinny_lds<...>", "pad_rows + pad_rows +
+ * dense_tiled<...>", ...), on aligned operands; with_workspace != 0 assumes the caller passes the workspace of
+ * mslk_amd_f8f8bf16_rowwise_workspace_bytes.  A dry run of the real dispatch code on the current device (or, with no GPU,
+ * for a whole MI355X): nothing is launched and no pointer is read.  Used by the tests to pin the shape classes of the
+ * benchmark configurations; no counterpart in the reference, whose dispatch is a table of tuned instances
+ * (csrc/gemm/ck/fp8_rowwise/fp8fp8bf16_rowwise_gemm.hip:158-468).  The returned string is thread-local and valid until
+ * the next call on the same thread.
+ */
+const char* mslk_amd_debug_dispatch_name(int64_t M, int64_t N, int64_t K, int bias_dtype, int y_dtype, int preshuffled,
+                                         int with_workspace);
+
+/*
  * Ceiling probes for the benchmark's roofline columns; no counterpart in the reference (its bench divides by fixed
  * peak figures, bench/gemm/gemm_bench.py:61-68) and not part of the product path.
  *   mslk_amd_debug_stream_read: `workgroups` x 256 lanes read `bytes` from `src` once and write nothing.  mode 0: 16-byte

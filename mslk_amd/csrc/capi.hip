@@ -419,6 +419,22 @@ int mslk_amd_debug_cast_e4m3fn(const float* in, int64_t n, void* out, void* stre
   return check_hip(launch_cast_e4m3fn(in, n, out, (hipStream_t)stream), "cast launch");
 }
 
+const char* mslk_amd_debug_dispatch_name(int64_t M, int64_t N, int64_t K, int bias_dtype, int y_dtype, int preshuffled,
+                                         int with_workspace) {
+  // Aligned stand-in pointers: the dry run dereferences nothing and launches nothing.
+  void* const fake = reinterpret_cast<void*>(uintptr_t(1) << 20);
+  thread_local char result[600];
+  const size_t wbytes = with_workspace ? mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K) : 0;
+  dispatch_probe_begin();
+  const int rc = rowwise_impl("debug_dispatch_name", y_dtype == MSLK_AMD_DTYPE_F16, preshuffled, fake, fake, (const float*)fake,
+                              (const float*)fake, bias_dtype ? fake : nullptr, bias_dtype, fake, M, N, K, wbytes ? fake : nullptr,
+                              wbytes, nullptr);
+  const char* text = dispatch_probe_end();
+  if (rc != 0) snprintf(result, sizeof(result), "error: %s", g_err);
+  else snprintf(result, sizeof(result), "%s", text[0] ? text : "nothing to launch");
+  return result;
+}
+
 int mslk_amd_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, void* stream) {
   if (mode != 0 && mode != 1) return fail("debug_stream_read: mode must be 0 (register loads) or 1 (LDS DMA loads)");
   if (bytes < 0 || bytes % (mode == 0 ? 16 : 1024) != 0) return fail("debug_stream_read: bytes must be a non-negative multiple of %d", mode == 0 ? 16 : 1024);

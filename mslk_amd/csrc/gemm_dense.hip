@@ -1,6 +1,9 @@
 // Dense f8f8bf16_rowwise for gfx950: LDS-tiled MFMA kernel (large shapes), a generic
 // any-shape kernel, and the zero-fill used for empty problems.
 #include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
 #include "gemm_tile.h"
 #include "kernels.h"
 
@@ -8,11 +11,39 @@ namespace mslk_amd {
 namespace {
 
 constexpr int kXcds = 8;      // MI355X: 8 accelerator dies, workgroups are dealt to them round-robin
-constexpr int kCus = 256;     // compute units of a whole MI355X; a 256 x 256 tile takes the whole LDS of one
+constexpr int kCus = 256;     // compute units of a whole MI355X (used when the device cannot be queried)
+
+struct DispatchProbe {
+  bool active = false;
+  char text[512] = "";
+};
+thread_local DispatchProbe g_probe;
+
+}  // namespace
+
+void dispatch_probe_begin() {
+  g_probe.active = true;
+  g_probe.text[0] = 0;
+}
+const char* dispatch_probe_end() {
+  g_probe.active = false;
+  return g_probe.text;
+}
+bool dispatch_probe_record(const char* fmt, ...) {
+  if (!g_probe.active) return false;
+  const size_t used = strlen(g_probe.text);
+  if (used > 0 && used + 4 < sizeof(g_probe.text)) strcat(g_probe.text, " + ");
+  const size_t at = strlen(g_probe.text);
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_probe.text + at, sizeof(g_probe.text) - at, fmt, ap);
+  va_end(ap);
+  return true;
+}
 
 // Compute units of the current device (a partitioned MI355X shows fewer than 256), as a multiple of the XCD count:
-// the number of persistent workgroups.  Queried once per device.
-int persistent_workgroups() {
+// the number of persistent workgroups and the CU count of the tile-shape thresholds.  Queried once per device.
+int device_compute_units() {
   static std::atomic<int> cached[64];   // zero-initialised; concurrent first calls store the same value
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return kCus;
@@ -25,6 +56,8 @@ int persistent_workgroups() {
   }
   return cus;
 }
+
+namespace {
 constexpr int kGroupM = 4;    // tiles of one XCD form kGroupM-row panels (L2 reuse of the WQ panel)
 
 // Workgroup id -> tile.  Consecutive workgroup ids land on different XCDs (each with a private
@@ -128,6 +161,8 @@ template <typename TS, bool PS>
 hipError_t launch_persistent_shape(const GemmProblem& p, int wgs, hipStream_t s) {
   constexpr int BM = TS::kBM, BN = TS::kBN;
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
+  if (dispatch_probe_record("dense_persistent<%d,%d>%s tiles=%d workgroups=%d", BM, BN, PS ? " preshuffled" : "", tiles_m * tiles_n, wgs))
+    return hipSuccess;
   switch (p.bias_dtype) {
     case 0: dense_persistent_kernel<TS, 0, PS><<<wgs, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
     case 1: dense_persistent_kernel<TS, 1, PS><<<wgs, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
@@ -142,6 +177,9 @@ hipError_t launch_tiled_shape(const GemmProblem& p, hipStream_t s) {
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const int grid = ((ntiles + kXcds - 1) / kXcds) * kXcds;
+  if (dispatch_probe_record("dense_tiled<%d,%d,waves=%dx%d,ring=%d>%s tiles=%d", BM, BN, TS::WM, TS::WN, TS::RING,
+                            PS ? " preshuffled" : "", ntiles))
+    return hipSuccess;
   switch (p.bias_dtype) {
     case 0: dense_tiled_kernel<TS, 0, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
     case 1: dense_tiled_kernel<TS, 1, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
@@ -234,7 +272,7 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // second launch, which picks smaller tiles for them (N = K = 8192, M = 2304: 160 -> 125 us; N = K = 4096, M = 4608:
   // 82 -> 62 us).
   {
-    const int wgs = persistent_workgroups();
+    const int wgs = device_compute_units();
     const int64_t tiles_n = (p.N + 255) / 256, tiles = (int64_t)((p.M + 255) / 256) * tiles_n;
     if (tiles > wgs) {
       const int64_t passes = (tiles + wgs - 1) / wgs;
@@ -253,7 +291,9 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
     }
   }
   // 256 x 256 tiles once they give most CUs work (one persistent workgroup per CU when there are more tiles than
-  // CUs); smaller tiles below that.
+  // CUs); smaller tiles below that.  Every tile-count threshold below was measured on a whole MI355X (256 CUs: 64, 128,
+  // 160, 192, 256 tiles) and is written as a fraction of the CU count of the device, so a partition scales them.
+  const int cus = device_compute_units();   // 256 on a whole MI355X; the thresholds below scale with a partition's CU count
   const int64_t big_tiles = (int64_t)((p.M + 255) / 256) * ((p.N + 255) / 256);
   // 128 x 128 tiles: with at most one tile per CU a workgroup gets the whole LDS for a five-deep ring (its step is
   // much shorter than a memory round trip); with more tiles two workgroups per CU hide each other's latency better.
@@ -262,11 +302,11 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // buffers) put the weight stream on two / four times as many CUs, still one workgroup per CU; the activations they
   // re-read come from L2.  Going narrower than one workgroup per CU was measured and is slower.
   if (p.w_preshuffled) {
-    if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, true>(p, persistent_workgroups(), s);
-    if (big_tiles >= 192) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
-    if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, true>(p, s);
-    if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, true>(p, s);
-    if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
+    if (big_tiles > cus) return launch_persistent_shape<TileShape<256, 256>, true>(p, cus, s);
+    if (big_tiles >= cus * 3 / 4) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
+    if (small_tiles <= cus / 4 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, true>(p, s);
+    if (small_tiles <= cus / 2 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, true>(p, s);
+    if (small_tiles <= cus) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
     return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
   }
   // M <= 64 on wide row-major weights (the caller sends M <= 8 to the weight-streaming kernel): the activation rows
@@ -280,7 +320,7 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
     if (p.M <= 32 || p.N <= 8192) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false>(p, s);
     return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false>(p, s);
   }
-  if (big_tiles > kCus) return launch_persistent_shape<TileShape<256, 256>, false>(p, persistent_workgroups(), s);
+  if (big_tiles > cus) return launch_persistent_shape<TileShape<256, 256>, false>(p, cus, s);
   // 128 x 256 tiles (wave tile 64 x 128, three ring buffers, one workgroup per CU) when they cover 160 ... 256 CUs in
   // a single pass and the 256 x 256 tiles would cover fewer than 160, or would leave their last row of tiles at most
   // half full -- fewer LDS bytes per MFMA than 128 x 128 tiles and half the row granularity of 256 x 256
@@ -289,13 +329,13 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   {
     const int64_t rows128 = (p.M + 127) / 128;
     const int64_t tiles12 = rows128 * ((p.N + 255) / 256);
-    if (tiles12 >= 160 && tiles12 <= kCus && (big_tiles < 160 || rows128 % 2 == 1))
+    if (tiles12 >= cus * 5 / 8 && tiles12 <= cus && (big_tiles < cus * 5 / 8 || rows128 % 2 == 1))
       return launch_tiled_shape<TileShape<128, 256, 2, 2, 3>, false>(p, s);
   }
   // Otherwise 256 x 256 tiles from 129 tiles on: the 128 x 256 tiles would then need two passes and the co-resident
   // 128 x 128 tiles more than two per CU (N = 6144, M = 1536: 144 tiles, K = 8192: 100.0 -> 87.1 us, K = 4096:
   // 48.9 -> 39.5 us).
-  if (big_tiles > 128) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  if (big_tiles > cus / 2) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
   // M > 64 with at most one 64 x 64 tile per CU: such tiles (four waves stacked along M, five ring buffers, two
   // workgroups per CU) wherever they cover at least as many CUs as the 128-row tiles below would, in a single pass:
   // rows 65 ... 128 then do not cost a second, half-empty 128-row tile's worth of activation traffic (N = K = 8192,
@@ -303,16 +343,17 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   if (p.M > 64 && p.N >= 1024) {
     const int64_t tiles64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
     const int64_t rows128 = (p.M + 127) / 128;
-    const int64_t tiles128 = small_tiles <= 64 ? rows128 * ((p.N + 31) / 32) : small_tiles <= 128 ? rows128 * ((p.N + 63) / 64) : small_tiles;
-    if (tiles64 <= kCus && tiles64 >= tiles128) return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false>(p, s);
+    const int64_t tiles128 = small_tiles <= cus / 4 ? rows128 * ((p.N + 31) / 32) : small_tiles <= cus / 2 ? rows128 * ((p.N + 63) / 64) : small_tiles;
+    if (tiles64 <= cus && tiles64 >= tiles128) return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false>(p, s);
   }
-  if (small_tiles <= 64 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false>(p, s);
-  if (small_tiles <= 128 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false>(p, s);
-  if (small_tiles <= 256) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false>(p, s);
+  if (small_tiles <= cus / 4 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false>(p, s);
+  if (small_tiles <= cus / 2 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false>(p, s);
+  if (small_tiles <= cus) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false>(p, s);
   return launch_tiled_shape<TileShape<128, 128>, false>(p, s);
 }
 
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s) {
+  if (dispatch_probe_record("generic_scalar")) return hipSuccess;
   const int64_t total = (int64_t)p.M * p.N;
   generic_kernel<<<(unsigned)((total + 255) / 256), 256, 0, s>>>(p);
   return hipGetLastError();
@@ -330,6 +371,7 @@ hipError_t launch_preshuffle_b(const void* src, void* dst, int64_t G, int64_t N,
 hipError_t launch_pad_rows(const uint8_t* src, uint8_t* dst, int64_t rows, int64_t K, int64_t Kp, hipStream_t s) {
   const int64_t chunks = rows * (Kp / 16);
   if (chunks <= 0) return hipSuccess;
+  if (dispatch_probe_record("pad_rows")) return hipSuccess;
   const int64_t want = (chunks + 255) / 256;
   pad_rows_kernel<<<(unsigned)(want > 65536 ? 65536 : want), 256, 0, s>>>(src, dst, chunks, (int)(Kp / 16), (int)K);
   return hipGetLastError();
@@ -337,6 +379,7 @@ hipError_t launch_pad_rows(const uint8_t* src, uint8_t* dst, int64_t rows, int64
 
 hipError_t launch_fill_zero_bf16(uint16_t* y, int64_t n, hipStream_t s) {
   if (n <= 0) return hipSuccess;
+  if (dispatch_probe_record("fill_zero")) return hipSuccess;
   const int64_t want = (n + 255) / 256;
   fill_zero_kernel<<<(unsigned)(want > 4096 ? 4096 : want), 256, 0, s>>>(y, n);
   return hipGetLastError();

@@ -175,6 +175,8 @@ __global__ __launch_bounds__(kWaves * 64) void skinny_kernel(GemmProblem p) {
 template <int MT, int NT, int U, bool PS = false, int kWaves = 8>
 hipError_t launch_cfg(const GemmProblem& p, hipStream_t s) {
   const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
+  if (dispatch_probe_record("skinny_registers<m_frags=%d,n_frags=%d,steps=%d>%s workgroups=%u", MT, NT, U, PS ? " preshuffled" : "", grid))
+    return hipSuccess;
   switch (p.bias_dtype) {
     case 0: skinny_kernel<MT, NT, U, kWaves, 0, PS><<<grid, kWaves * 64, 0, s>>>(p); break;
     case 1: skinny_kernel<MT, NT, U, kWaves, 1, PS><<<grid, kWaves * 64, 0, s>>>(p); break;
@@ -367,6 +369,8 @@ __global__ __launch_bounds__(512) void skinny_lds_kernel(GemmProblem p) {
 template <int MT, int NT, int U, bool PS = false>
 hipError_t launch_lds(const GemmProblem& p, hipStream_t s) {
   const unsigned grid = (unsigned)((p.N + NT * 16 - 1) / (NT * 16));
+  if (dispatch_probe_record("skinny_lds<m_frags=%d,n_frags=%d,steps=%d>%s workgroups=%u", MT, NT, U, PS ? " preshuffled" : "", grid))
+    return hipSuccess;
   switch (p.bias_dtype) {
     case 0: skinny_lds_kernel<MT, NT, U, 0, PS><<<grid, 512, 0, s>>>(p); break;
     case 1: skinny_lds_kernel<MT, NT, U, 1, PS><<<grid, 512, 0, s>>>(p); break;

@@ -62,6 +62,16 @@ struct GemmProblem {
   int w_preshuffled;  // 1: WQ is in the blocked layout [N/16][K/64][4][16][16 B] (N % 16 == 0, K % 64 == 0)
 };
 
+// Dry run of the shape dispatch (mslk_amd_debug_dispatch_name): between dispatch_probe_begin() and dispatch_probe_end()
+// on the calling thread every GEMM launcher records the kernel it would launch (name, tile shape, grid) and launches
+// nothing -- the recorded choice is made by the very code that makes the real one.
+void dispatch_probe_begin();
+const char* dispatch_probe_end();                       // "a + b" when the dispatch would issue several launches
+bool dispatch_probe_record(const char* fmt, ...);       // false when no dry run is active on this thread
+// Compute units of the current device, rounded down to a multiple of the XCD count (256 on a whole MI355X, also
+// when no device can be queried); the tile-shape thresholds and the persistent grid both use it.
+int device_compute_units();
+
 // Shape classes; each returns hipErrorInvalidValue when the shape is outside what it supports.
 bool dense_tiled_supports(const GemmProblem& p);
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s);

@@ -144,3 +144,54 @@ def test_product_package_never_imports_the_oracle():
             if f.endswith((".py", ".hip", ".h")):
                 text = open(os.path.join(dirpath, f)).read()
                 assert "import oracle" not in text and "from oracle" not in text and "liboracle" not in text, f
+
+
+# (M, N, K, bias code, y dtype code, pre-shuffled, with workspace) -> the kernel the dense entry points pick on a whole
+# MI355X.  The thresholds behind these choices were measured; an edit that moves one of the benchmark configurations (or
+# a neighbouring shape class) to another kernel has to change this table knowingly.
+DISPATCH_TABLE = [
+    ((1024, 1024, 1024, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=256"),                       # cfg0
+    ((4096, 4096, 4096, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256"),                     # cfg1
+    ((8192, 28672, 4096, 2, 0, 0, 1), "dense_persistent<256,256> tiles=3584 workgroups=256"),                # cfg2
+    ((1, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),                 # cfg3, M = 1
+    ((4, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),
+    ((16, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> tiles=256"),
+    ((64, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,32,waves=4x1,ring=6> tiles=256"),
+    ((16, 8192, 8192, 0, 0, 1, 1), "skinny_lds<m_frags=1,n_frags=2,steps=2> preshuffled workgroups=256"),    # cfg3 on blocked weights
+    ((64, 8192, 8192, 0, 0, 1, 1), "skinny_lds<m_frags=4,n_frags=2,steps=1> preshuffled workgroups=256"),
+    ((64, 4096, 14336, 0, 0, 0, 1), "skinny_lds<m_frags=4,n_frags=1,steps=1> workgroups=256"),
+    ((8, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),                  # last M of the streaming kernel on wide weights
+    ((9, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> tiles=256"),
+    ((3, 1000, 272, 0, 0, 0, 1), "skinny_registers<m_frags=1,n_frags=1,steps=8> workgroups=63"),              # K % 1024 != 0
+    ((8192, 8192, 8192, 0, 0, 0, 1), "dense_persistent<256,256> tiles=1024 workgroups=256"),
+    ((2304, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256 + dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
+    ((2048, 4096, 4096, 0, 0, 0, 1), "dense_tiled<128,256,waves=2x2,ring=3> tiles=256"),
+    ((1536, 6144, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=144"),
+    ((512, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,128,waves=2x2,ring=5> tiles=256"),
+    ((256, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
+    ((128, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=256"),
+    ((4096, 8192, 4096, 0, 0, 0, 1), "dense_persistent<256,256> tiles=512 workgroups=256"),
+    ((4096, 4096, 4096, 0, 1, 1, 1), "dense_tiled<256,256,waves=2x2,ring=0> preshuffled tiles=256"),
+    ((4096, 4096, 4100, 0, 0, 0, 1), "pad_rows + pad_rows + dense_tiled<256,256,waves=2x2,ring=0> tiles=256"),
+    ((4096, 4096, 4100, 0, 0, 0, 0), "generic_scalar"),
+    ((5, 7, 0, 0, 0, 0, 1), "fill_zero"),
+    ((0, 16, 16, 0, 0, 0, 1), "nothing to launch"),
+]
+
+
+@pytest.mark.parametrize("args,want", DISPATCH_TABLE)
+def test_dispatch_of_the_dense_entry_points_is_pinned(args, want):
+    """mslk_amd_debug_dispatch_name runs the real dispatch code as a dry run (nothing is launched, no GPU needed: without
+    one it assumes the 256 compute units of a whole MI355X)."""
+    from mslk_amd import _lib
+    got = _lib.lib().mslk_amd_debug_dispatch_name(*args).decode()
+    assert got == want
+
+
+def test_dispatch_dry_run_reports_argument_errors_and_leaves_no_state():
+    from mslk_amd import _lib
+    L = _lib.lib()
+    assert L.mslk_amd_debug_dispatch_name(16, 24, 64, 0, 0, 1, 1).decode().startswith("error: ")   # N % 16 != 0 for blocked weights
+    assert L.mslk_amd_debug_dispatch_name(-1, 16, 16, 0, 0, 0, 1).decode().startswith("error: ")
+    # the dry run is over when the call returns: a real call would launch again (here: rejected for its null output first)
+    assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 0, None, 4, 4, 16, None, 0, None) != 0

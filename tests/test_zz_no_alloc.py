@@ -8,6 +8,8 @@ import pytest
 import torch
 
 from mslk_amd import _lib
+from oracle import fp8_rowwise_oracle as O
+from tests.helpers import assert_gemm_close
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -53,9 +55,23 @@ def test_static_scratch_matches_the_workspace_entry_point_on_two_calls():
         print(f"static scratch case {i}: M={M} N={N} K={K}", flush=True)
         ops = _operands(M, N, K, seed=50 + i)
         want = _with_workspace(*ops, M, N, K)
-        got = _static(*ops, M, N, K)
         torch.cuda.synchronize()
+        allocated, free = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+        L = _lib.lib()
+        y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+        allocated_with_y, free_with_y = torch.cuda.memory_allocated(), torch.cuda.mem_get_info()[0]
+        _lib.check(L.mslk_amd_f8f8bf16_rowwise_static_scratch(*(t.data_ptr() for t in ops[:4]), ops[4].data_ptr(), 2, y.data_ptr(),
+                                                              M, N, K, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        # nothing was allocated or freed by the call: neither through torch's allocator nor behind its back on the device
+        assert torch.cuda.memory_allocated() == allocated_with_y and torch.cuda.mem_get_info()[0] == free_with_y
+        assert allocated_with_y >= allocated and free_with_y <= free
+        got = y
         assert torch.equal(got.view(torch.int16).cpu(), want.view(torch.int16).cpu()), f"case {i}: outputs differ"
+        # and both agree with the oracle (the comparison above is one HIP path against another)
+        xq, wq, xs, ws, bias = (t.cpu() for t in ops)
+        ref = O.dequant_matmul(xq.view(torch.float8_e4m3fn), wq.view(torch.float8_e4m3fn), xs, ws, bias.float())
+        assert_gemm_close(got, ref, f"static scratch case {i}")
 
 
 def test_static_scratch_aligned_shapes_do_not_need_the_array():
@@ -78,3 +94,30 @@ def test_static_scratch_rejects_what_does_not_fit():
     assert rc != 0
     msg = L.mslk_amd_last_error().decode()
     assert "static scratch" in msg and "workspace" in msg
+
+
+def test_static_scratch_under_graph_capture_and_replay():
+    """The entry point is meant for code under HIP graph capture.  The address of the library's array is looked up on the
+    first call on a device (hipGetSymbolAddress, not a stream operation); the calls above have done that, and a caller
+    that captures should make one call -- any shape that needs the copies -- outside capture first, as here.  A K % 16 != 0
+    shape is captured (two copy kernels + the GEMM), replayed with eager work between the replays, and every replay is
+    compared with the eager result."""
+    M, N, K = 40, 520, 1001
+    ops = _operands(M, N, K, seed=91)
+    eager = _static(*ops, M, N, K)                      # also primes the symbol lookup outside capture
+    torch.cuda.synchronize()
+    L = _lib.lib()
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _lib.check(L.mslk_amd_f8f8bf16_rowwise_static_scratch(*(t.data_ptr() for t in ops[:4]), ops[4].data_ptr(), 2, y.data_ptr(),
+                                                              M, N, K, torch.cuda.current_stream().cuda_stream))
+    other = _operands(17, 264, 200, seed=92)
+    for _ in range(3):
+        y.fill_(3.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y.view(torch.int16), eager.view(torch.int16))
+        _static(*other, 17, 264, 200)                  # eager work on the same scratch array between the replays
+        torch.cuda.synchronize()
