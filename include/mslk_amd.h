@@ -154,6 +154,9 @@ size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K
  * (M + N) * round_up(K, 16) > MSLK_AMD_STATIC_SCRATCH_BYTES, are rejected with an error.  The array needs no
  * initialisation (the copies overwrite every byte they later read), but all calls on one GPU share it: calls that
  * overlap on one GPU (different streams, or threads) race.  Shapes that need no copies never touch the array.
+ * The first call on a device that needs the copies looks the array's address up (hipGetSymbolAddress; not a stream
+ * operation) and is also the moment HIP commits the array's device memory; a caller that captures graphs or measures
+ * memory makes that first call outside the capture / before the measurement.
  */
 #define MSLK_AMD_STATIC_SCRATCH_BYTES ((size_t)32 << 20)
 int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, const float* x_scale, const float* w_scale,

@@ -37,6 +37,17 @@ __device__ __forceinline__ uint32_t cvt_pk_e4m3fn(float a, float b) {
 
 #define MSLK_AMD_DEVINL __device__ __forceinline__
 
+// 8-byte store of quantized codes, written through to memory at system scope (sc1) instead of being left dirty in the
+// L2 of the XCD that produced them or streamed past the caches (nt).  A write-through leaves nothing to flush when the
+// kernel ends (plain stores cost the row quantizer 1.6 us at 4096 x 4096) and, unlike a streaming store, leaves the
+// codes in the memory-side cache, where the GEMM that consumes them finds them: quantize -> GEMM at 4096^3 takes
+// 60.6 us with nt stores, 58.9 with plain ones and 57.7 with these; the quantizer alone 12.4 / 14.0 / 12.5 us.
+// Written as an instruction because the compiler offers no spelling for the scope bits of a plain store; an 8-byte store
+// needs no wait states behind it, and the "memory" clobber keeps it ordered with the surrounding accesses.
+__device__ __forceinline__ void store8_write_through(void* dst, v2i v) {
+  asm volatile("global_store_dwordx2 %0, %1, off sc1" : : "v"(dst), "v"(v) : "memory");
+}
+
 // Two fp32 -> packed bf16 (lo = a, hi = b), round to nearest even, by the hardware conversion.
 typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef float f32x2_t __attribute__((ext_vector_type(2)));

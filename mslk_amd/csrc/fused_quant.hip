@@ -141,10 +141,11 @@ MSLK_AMD_DEVINL void row_scales(uint32_t max_bits, const float* scale_ub, float&
 MSLK_AMD_DEVINL uint2 quantize8_saturating(const float (&y)[8], float s) {
   float f[8];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) f[i] = __builtin_fminf(__builtin_fmaxf(y[i] * s, -kMaxFp8), kMaxFp8);
+  for (int i = 0; i < 8; ++i) f[i] = __builtin_amdgcn_fmed3f(y[i] * s, -kMaxFp8, kMaxFp8);   // clamp; a NaN comes out as -448, as from fmin(fmax())
+  // within +-448 the hardware conversion alone gives the codes (no NaN / overflow fix-up to apply)
   uint2 r;
-  r.x = cvt_pk_e4m3fn(f[0], f[1]) | (cvt_pk_e4m3fn(f[2], f[3]) << 16);
-  r.y = cvt_pk_e4m3fn(f[4], f[5]) | (cvt_pk_e4m3fn(f[6], f[7]) << 16);
+  r.x = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false), true);
+  r.y = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false), true);
   return r;
 }
 
@@ -197,7 +198,7 @@ __global__ __launch_bounds__(256) void fused_quant_vec_kernel(FusedQuantArgs p) 
       const int vec = i * TEAM + lane;
       if (vec < nvec) {
         const uint2 q = quantize8_saturating(cache[i], s);
-        __builtin_nontemporal_store(v2i{(int)q.x, (int)q.y}, reinterpret_cast<v2i*>(out_row + vec));
+        store8_write_through(reinterpret_cast<v2i*>(out_row + vec), v2i{(int)q.x, (int)q.y});
       }
     }
   } else {
@@ -205,7 +206,7 @@ __global__ __launch_bounds__(256) void fused_quant_vec_kernel(FusedQuantArgs p) 
       float y[8];
       produce8<OP, DTYPE>(r, vec, y);
       const uint2 q = quantize8_saturating(y, s);
-      __builtin_nontemporal_store(v2i{(int)q.x, (int)q.y}, reinterpret_cast<v2i*>(out_row + vec));
+      store8_write_through(reinterpret_cast<v2i*>(out_row + vec), v2i{(int)q.x, (int)q.y});
     }
   }
 }

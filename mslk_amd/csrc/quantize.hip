@@ -29,9 +29,7 @@ namespace {
 template <int DTYPE> struct Vec8 { uint4 w; };          // 8 x 16-bit
 template <> struct Vec8<2> { uint4 lo, hi; };           // 8 x fp32
 
-MSLK_AMD_DEVINL void store8_stream(uint2* dst, uint2 val) {
-  __builtin_nontemporal_store(v2i{(int)val.x, (int)val.y}, reinterpret_cast<v2i*>(dst));
-}
+MSLK_AMD_DEVINL void store8_stream(uint2* dst, uint2 val) { store8_write_through(dst, v2i{(int)val.x, (int)val.y}); }
 
 template <int DTYPE>
 MSLK_AMD_DEVINL Vec8<DTYPE> load_vec8(const void* row_ptr, int vec_idx) {
@@ -79,7 +77,12 @@ MSLK_AMD_DEVINL uint32_t finish_absmax_bits(uint32_t m) {
 // with rcp = fl32(1 / factor) -- a handful of instructions instead of a division sequence.  The e4m3 codes are those of the
 // IEEE division for every 16-bit element not above a 16-bit row maximum of at least 2^-64 (checked exhaustively on the
 // CPU, tests/test_oracle.py); the caller passes rcp = 0 for every other row, which then divides.
-template <int DTYPE, bool TRITON>
+// clamp(v, -448, 448) in one instruction (the median of the three; a NaN comes out as -448, like fmin(fmax(v, -448), 448))
+MSLK_AMD_DEVINL float clamp448(float v) { return __builtin_amdgcn_fmed3f(v, -448.0f, 448.0f); }
+
+// PLAIN (torch arithmetic only): the caller knows that no product of the row exceeds 448 (1 + 2^-22) and none is NaN -- a
+// finite row maximum that scale_ub has not cut -- so the hardware conversion alone gives the codes.
+template <int DTYPE, bool TRITON, bool PLAIN = false>
 MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float factor, float rcp = 0.f) {
   float f[8];
   if constexpr (DTYPE == 2) {
@@ -101,15 +104,27 @@ MSLK_AMD_DEVINL uint2 quantize_vec8(const Vec8<DTYPE>& v, float factor, float rc
         const float q0 = f[i] * rcp;
         const float e = __builtin_fmaf(-q0, factor, f[i]);
         const float q = e == 0.f ? q0 : __builtin_fmaf(e, rcp, q0);
-        f[i] = __builtin_fminf(__builtin_fmaxf(q, -448.0f), 448.0f);
+        f[i] = clamp448(q);
       }
     } else {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) f[i] = __builtin_fminf(__builtin_fmaxf(f[i] / factor, -448.0f), 448.0f);
+      for (int i = 0; i < 8; ++i) f[i] = clamp448(f[i] / factor);
     }
+    // Everything is within +-448 now (a NaN quotient came out of the clamp as -448, as it did with a max / min pair), so
+    // the plain hardware conversion gives the codes; the fix-up for magnitudes beyond 464 has nothing left to do.
+    uint2 r;
+    r.x = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false), true);
+    r.y = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false), true);
+    return r;
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = f[i] * factor;
+    if constexpr (PLAIN) {
+      uint2 r;
+      r.x = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], 0, false), true);
+      r.y = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], 0, false), true);
+      return r;
+    }
   }
   uint2 r;
   r.x = cvt_pk_e4m3fn(f[0], f[1]) | (cvt_pk_e4m3fn(f[2], f[3]) << 16);
@@ -206,10 +221,20 @@ __global__ __launch_bounds__(256) void quantize_rows_vec_kernel(
   if (!live) {   // an empty row quantizes to zero codes
     for (int idx = lane; idx < nvec; idx += TEAM) store8_stream(out_row + idx, make_uint2(0u, 0u));
   } else if constexpr (CACHED) {
+    // torch arithmetic: a row with a finite maximum that scale_ub did not cut needs no NaN / overflow fix-up behind the
+    // hardware conversion (uniform over the team)
+    if (!TRITON && scale_ub == nullptr && amax < __builtin_inff()) {
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int idx = i * TEAM + lane;
-      if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(cache[i], inv, rcp));
+      for (int i = 0; i < NV; ++i) {
+        const int idx = i * TEAM + lane;
+        if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON, !TRITON>(cache[i], inv, rcp));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int idx = i * TEAM + lane;
+        if (idx < nvec) store8_stream(out_row + idx, quantize_vec8<DTYPE, TRITON>(cache[i], inv, rcp));
+      }
     }
   } else {
     for (int idx = lane; idx < nvec; idx += TEAM)
