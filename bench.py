@@ -323,7 +323,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", default="",
-                    help="helper: run only this piece (gemm|gemm-timed|power|quantize|decode|cfg2|grouped|traffic|vendor|ceilings) and exit")
+                    help="helper: run only this piece (gemm|gemm-timed|power|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|ceilings) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -533,6 +533,29 @@ def main():
         p_ms = _median_events_ms(path_step, 50)
         extras["quantize_plus_gemm_cfg1"] = {"ms": p_ms, "TFLOPs": flops / (p_ms * 1e-3) / 1e12}
     del xsets
+
+    # ---------------------------------------------------------------- decode, eager or graph launches only (for a kernel trace)
+    if args.only in ("decode-eager", "decode-graph"):
+        # The same decode GEMMs launched one by one or replayed from ONE HIP graph, and nothing else: under
+        # `rocprofv3 --kernel-trace --stats` the two runs give each kernel's duration in either mode, to set beside the
+        # per-launch times (M = 1, 16 and 64 run three different kernels, so the statistics keep them apart).
+        wq3, ws3 = mslk_amd.quantize_fp8_row(W.cfg3_weight().to(dev), use_triton=False)
+        wsets = [wq3.clone() for _ in range(6)]
+        res = {}
+        for Md in (1, 16, 64):
+            xq3, xs3 = mslk_amd.quantize_fp8_row(W.cfg3_activations(Md).to(dev), use_triton=False)
+            y3 = torch.empty(Md, 8192, dtype=torch.bfloat16, device=dev)
+
+            def dec_step(i):
+                api.gemm(xq3, wsets[i % len(wsets)], xs3, ws3, y3)
+
+            if args.only == "decode-eager":
+                _settle(dec_step, 20.0)
+                res[f"M{Md}"] = {"ms_per_launch": _median_events_ms(dec_step, 60)}
+            else:
+                res[f"M{Md}"] = {"ms_per_launch": _graph_ms(dec_step, 60, repeats=12)}
+        print(json.dumps({args.only: res}))
+        return
 
     # ---------------------------------------------------------------- decode sweep (cfg3)
     if (not args.no_extras and args.only == "") or args.only == "decode":
