@@ -146,8 +146,8 @@ def _quantize_fp8_row_fake(a, scale_ub=None, zero_start_index_M=None, use_triton
 
 
 def _quantize_fp8_per_row_gpu(input, bs=None, scale_ub=None, output_dtype=None, stochastic_rounding=False):
-    """GPU kernel of `mslk::quantize_fp8_per_row`: row amax, scale = amax / 448, cast to e4m3fn, with the bits of the
-    reference's torch emulation (fp8_quantize.py:356-378)."""
+    """GPU kernel of `mslk::quantize_fp8_per_row` (a convenience operator, not one of the reference's): row amax,
+    scale = amax / 448, cast to e4m3fn, with the bits of the reference's torch emulation (fp8_quantize.py:356-378)."""
     if bs is not None:
         raise NotImplementedError("quantize_fp8_per_row: `bs` is not supported")
     if stochastic_rounding:
@@ -162,10 +162,13 @@ def _quantize_fp8_per_row_fake(input, bs=None, scale_ub=None, output_dtype=None,
             torch.empty(input.shape[:-1], dtype=torch.float32, device=input.device))
 
 
-# Registered with the low-level library API (a few microseconds of dispatch per call); GPU kernels only.  The names and
-# schemas are the ones callers of the reference use: `triton::quantize_fp8_row` is what its
-# torch.library.custom_op (fp8_quantize.py:319-328) defines, so a traced or compiled caller of
-# torch.ops.triton.quantize_fp8_row lands here; when the reference defined the op first only its GPU kernel is replaced.
+# Registered with the low-level library API (a few microseconds of dispatch per call); GPU kernels only.
+# `triton::quantize_fp8_row` is the operator the reference's torch.library.custom_op (fp8_quantize.py:319-328) defines,
+# with its schema and defaults, so a traced or compiled caller of torch.ops.triton.quantize_fp8_row lands here.  When the
+# reference defined the op first, only its GPU kernel is replaced; the other way round does not work (the reference's
+# custom_op would meet an existing definition), so a process that uses both imports the reference's module first.
+# `mslk::quantize_fp8_per_row` has no counterpart in the reference tree: it is a convenience operator under the name the
+# path is known by (the legacy FBGEMM operator's signature), always with the torch branch's arithmetic.
 _library = torch.library.Library("mslk", "FRAGMENT")
 _triton_library = torch.library.Library("triton", "FRAGMENT")
 _QUANTIZE_ROW_SCHEMA = ("quantize_fp8_row(Tensor a, Tensor? scale_ub=None, Tensor? zero_start_index_M=None, "
