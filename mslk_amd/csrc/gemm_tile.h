@@ -75,6 +75,24 @@ typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
 // read-back values in accumulator registers, all of which hold the tile, and spills part of it.  The compiler does
 // not see a store here, so the wait states the hardware needs between a store of more than 8 bytes and a vector
 // instruction that overwrites its data registers (the allocator reuses them at once) are part of the statement.
+//
+// Rules for the statements in this file that the compiler cannot look into (each was learnt from a wrong result or a fault):
+//   1. An instruction written by hand gets the wait states the hardware asks for INSIDE its statement (the s_nop 1 below,
+//      the s_nop 0 between the M0 write and the load in dma16): the hazard pass does not see through it.
+//   2. A memory READ written by hand must keep its destination registers live until a wait inside the same statement:
+//      the allocator otherwise hands them out again while the load is in flight, and the late write-back lands in a live
+//      value (an address, once: a memory fault).  This file has no such read -- dma16 has no register destination.
+//   3. What the compiler does not know to be in flight it does not wait for: every read of bytes copied by dma16 sits
+//      behind an explicit s_waitcnt vmcnt in wait_and_barrier() / wait_vmcnt0().
+//   4. Accumulator registers read by hand (v_accvgpr_read_b32 in the epilogue) follow a fixed 48 wait states behind the
+//      last MFMA of the K loop.
+// Which test fails when a rule is broken (all compare integer-valued products bit for bit): store16_stream and the
+// accumulator reads -- tests/test_gemm_gpu.py::test_exact_on_full_256_tiles (one tile per workgroup, fused and plain
+// epilogue, both output types, both bias types), tests/test_exact_paths_gpu.py::test_persistent_workgroups_exact (epilogue
+// behind the next tile's first loads), ::test_tensorlist_grouped_exact / ::test_stacked_and_offsets_over_m_exact (ragged and
+// interleaved epilogues); dma16 and the load waits -- every test of tests/test_exact_paths_gpu.py (each tile shape and
+// ring depth has a case) and tests/test_preshuffle_gpu.py; graph replays that must repeat the eager bits --
+// tests/test_gemm_gpu.py::test_hip_graph_capture_and_replay, tests/test_grouped_mm_gpu.py::test_graph_replay_follows_device_side_group_sizes.
 MSLK_AMD_DEVINL void store16_stream(uint16_t* dst, uint4 val) {
   const v4i v = {(int)val.x, (int)val.y, (int)val.z, (int)val.w};
   asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" : : "v"(dst), "v"(v) : "memory");
@@ -314,10 +332,7 @@ struct GemmTile {
 #pragma unroll
     for (int tn = 0; tn < TS::FN - 1; ++tn) {
       // Issue order inside a group: the read of the next WQ fragment follows the first MFMA, the DMA
-      // loads follow the last MFMAs, one each.  Every DMA sits in the shadow of an MFMA, and the
-      // LDS reads issued before it are at least four MFMAs old: the compiler orders all earlier LDS
-      // reads before a DMA write (it cannot see that the buffers are disjoint), so a DMA right
-      // behind a fresh read would stall on that read's latency.
+      // loads follow the last MFMAs, one each, so that every DMA is issued in the shadow of an MFMA.
       v8i wf_next;
 #pragma unroll
       for (int tm = 0; tm < TS::FM; ++tm) {
