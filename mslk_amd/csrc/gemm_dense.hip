@@ -112,7 +112,7 @@ template <typename TS, int BIAS, bool PS>
 __global__ __launch_bounds__(TS::NTHREADS) void dense_persistent_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   static_assert(TS::RING == 0 && TS::NTHREADS == 256, "two-plus-three buffer tiles with four waves");
   constexpr int BM = TS::kBM, BN = TS::kBN;
-  using Tile = GemmTile<TS, BIAS, PS>;
+  using Tile = GemmTile<TS, BIAS, PS, false, 0>;   // many tiles per XCD share every XQ line: one step ahead is enough
   // The epilogue parks its transposes in the two buffers the next tile's prologue does not fill.
   static_assert(2 * Tile::EPI_WAVE_BYTES <= TS::A_BYTES && 2 * Tile::EPI_WAVE_BYTES <= TS::B_BYTES, "transpose buffers fit");
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];

@@ -129,7 +129,9 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* base, uint32_t off, char* lds_wave_bas
 // MFMA operand read it (reference: mslk/quantize/shuffle.py:182-246).  One DMA then moves one block
 // (1 KiB contiguous in HBM and in LDS), the WQ fragment read is lane-linear, and both operands give
 // lane (i, g) the k bytes [16 g, 16 g + 16) and [64 + 16 g, 64 + 16 g + 16) of row i.
-template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false>
+// XQ_EARLY: how many of the LA loads of an XQ tile are issued two K steps ahead instead of one (two-plus-three buffers;
+// see step()).
+template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false, int XQ_EARLY = TS::LA / 2>
 struct GemmTile {
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
@@ -191,8 +193,12 @@ struct GemmTile {
   }
   // Ragged tiles: a wave whose share of the XQ tile (8 * LA consecutive rows) starts beyond the valid rows fetches
   // nothing -- nobody multiplies those rows (one wave-uniform branch for the wave's loads of a step).
-  MSLK_AMD_DEVINL void issue_a_live(char* abuf, int k0) {
-    if (wave_id() * TS::LA * 8 < a_rows) issue_a_all(abuf, k0);
+  MSLK_AMD_DEVINL void issue_a_live(char* abuf, int k0, int lo = 0, int hi = TS::LA) {
+    if (wave_id() * TS::LA * 8 < a_rows) {
+#pragma unroll
+      for (int i = 0; i < TS::LA; ++i)
+        if (i >= lo && i < hi) issue_a(abuf, k0, i);
+    }
   }
   MSLK_AMD_DEVINL void issue_b_all(char* bbuf, int k0) {
 #pragma unroll
@@ -288,47 +294,69 @@ struct GemmTile {
   }
 
   // One K step of MFMAs on the WQ tile in `b_cur`; xf / wf0 (the step's XQ fragments and WQ fragment 0)
-  // are already in registers.  The step is software-pipelined across the workgroup barrier and the
-  // weight stream runs two steps ahead:
-  //   * DMA_A / DMA_B: the global -> LDS loads of the XQ tile of the NEXT step (byte offset k_a, buffer
-  //     `a_nxt`) and of the WQ tile of the step AFTER it (byte offset k_b, buffer `b_far`) are issued
-  //     between the MFMA groups of the first half of the step, XQ first, so that their issue cost hides
-  //     under matrix work.  Weights are the cold stream (read once from HBM); giving them two steps to
-  //     land keeps twice as many bytes in flight per CU as a plain double buffer.
+  // are already in registers.  The step is software-pipelined across the workgroup barrier; the weight
+  // stream runs two steps ahead, the activation stream one to two:
+  //   * DMA_B: the global -> LDS loads of the WQ tile two steps on (byte offset k_b, buffer `b_far`) are
+  //     issued between the MFMA groups in front of the barrier, so that their issue cost hides under
+  //     matrix work.
   //   * NEXT: before the last MFMA group the wave waits for everything but the WQ loads it issued in this
   //     step, and for all its LDS reads, and passes the barrier (after which `a_nxt` and `b_nxt` are
   //     complete and nobody reads `b_cur` any more).  The operands of the last group are in registers;
   //     each XQ fragment is re-loaded from `a_nxt` right after the MFMA that used it last, so the barrier
   //     and the LDS latency overlap with matrix work and the following step starts with its first
   //     fragments already on their way.
-  // In the symmetric ring (TileShape::RING) the XQ loads go to `a_dst` != `a_nxt` as well, and PENDING, the
-  // number of this wave's youngest loads that may still be in flight at the barrier, covers RING - 2 steps.
+  //   * NA_TAIL (two-plus-three buffers): the first NA_TAIL loads of the XQ tile two steps on (byte offset
+  //     k_a_tail) go into `a_tail_dst`, the buffer THIS step's XQ fragments came from: they have been in
+  //     registers since the previous step, and once the barrier of this step is passed every wave has them,
+  //     so the loads follow the barrier, spread over the MFMAs of the last group.  They are then a whole step
+  //     old at the barrier that needs them; a load issued in front of the barrier, as the WQ loads are, has
+  //     to go to the other buffer and is less than a step old when it is needed -- less than the latency of
+  //     a line that misses the L2, which is what a tile sees whose XQ rows few other tiles of its XCD share.
+  //     All loads behind the barrier is too many: the four waves pass it together and their loads then queue
+  //     in front of the MFMAs (measured: 2 - 4 % slower on large shapes); half and half costs nothing there.
+  //   * NA_HEAD: the last NA_HEAD loads of the XQ tile ONE step on (byte offset k_a) go into `a_dst` in front
+  //     of the WQ loads.
+  //   * Symmetric ring (TileShape::RING): NA_HEAD = LA, all XQ loads go with the WQ loads in front of the barrier
+  //     into `a_dst` != `a_nxt`, and PENDING, the number of this wave's youngest loads that may still be in
+  //     flight at the barrier, covers RING - 2 steps.
   // FMV < FM: a ragged tile, only the first FMV m fragments of every wave hold valid rows -- see step_rows().
-  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING, int FMV = TS::FM>
+  template <int NA_HEAD, bool DMA_B, bool NEXT, int PENDING, int FMV = TS::FM, int NA_TAIL = 0>
   MSLK_AMD_DEVINL void step(const char* b_cur, char* a_dst, const char* a_nxt, const char* b_nxt, char* b_far, int k_a,
-                            int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
+                            int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0, char* a_tail_dst = nullptr,
+                            int k_a_tail = 0) {
+    static_assert(NA_HEAD >= 0 && NA_TAIL >= 0 && NA_HEAD <= TS::LA && NA_TAIL <= TS::LA && (NA_TAIL == 0 || NEXT), "XQ loads of a step");
     if constexpr (FMV < TS::FM) {
-      step_rows<DMA_A, DMA_B, NEXT, PENDING, FMV>(b_cur, a_dst, a_nxt, b_nxt, b_far, k_a, k_b, acc, xf, wf0);
+      step_rows<NA_HEAD, DMA_B, NEXT, PENDING, FMV, NA_TAIL>(b_cur, a_dst, a_nxt, b_nxt, b_far, k_a, k_b, acc, xf, wf0, a_tail_dst, k_a_tail);
       return;
     }
     v8i wf_last;
-    step_head<DMA_A, DMA_B>(b_cur, a_dst, b_far, k_a, k_b, acc, xf, wf0, wf_last);
-    step_tail<NEXT, PENDING>(a_nxt, b_nxt, acc, xf, wf0, wf_last);
+    step_head<NA_HEAD, DMA_B>(b_cur, a_dst, b_far, k_a, k_b, acc, xf, wf0, wf_last);
+    step_tail<NEXT, PENDING, NA_TAIL>(a_nxt, b_nxt, acc, xf, wf0, wf_last, a_tail_dst, k_a_tail);
   }
 
   // The part of a full-tile K step in front of its barrier: every n fragment but the last, with the step's DMA loads.
   // Leaves the last WQ fragment of the step in `wf_last`.
-  template <bool DMA_A, bool DMA_B>
+  template <int NA_HEAD, bool DMA_B>
   MSLK_AMD_DEVINL void step_head(const char* b_cur, char* a_dst, char* b_far, int k_a, int k_b, v4f (&acc)[TS::FN][TS::FM],
                                  v8i (&xf)[TS::FM], const v8i& wf0, v8i& wf_last) {
     constexpr int HALF = TS::FN / 2;
-    static_assert((TS::LA + TS::LB) % HALF == 0, "DMA loads spread evenly over the first half");
-    constexpr int NDMA = (TS::LA + TS::LB) / HALF;   // DMA loads per MFMA group
+    constexpr int NA = NA_HEAD, NB = DMA_B ? TS::LB : 0;   // the step's loads: the last NA of the XQ tile's first, then WQ
+    constexpr int ND = NA + NB, GD = TS::FN - 1;
+    constexpr int NDMA = (ND + HALF - 1) / HALF;                      // DMA loads per MFMA group (first half only)
     constexpr int PER_SLOT = (NDMA + TS::FM - 1) / TS::FM;            // 1 unless the tile has few MFMAs per group
-    constexpr int SLOTS = (NDMA + PER_SLOT - 1) / PER_SLOT;          // MFMA slots of a group that carry loads
+    constexpr int SLOTS = PER_SLOT > 0 ? (NDMA + PER_SLOT - 1) / PER_SLOT : 0;   // MFMA slots of a group that carry loads
+    constexpr bool SPREAD = PER_SLOT <= 1 && ND <= GD * TS::FM;
+    static_assert(SPREAD || ND % HALF == 0, "DMA loads spread evenly over the first half");
     const FragOff fo = frag_off();
     const char* b_tile = b_tile_of(b_cur);
     v8i wf = wf0;
+    auto issue = [&](int q) {
+      if (q < NA) {
+        if constexpr (NA > 0) issue_a(a_dst, k_a, TS::LA - NA + q);
+      } else {
+        if constexpr (DMA_B) issue_b(b_far, k_b, q - NA);
+      }
+    };
 #pragma unroll
     for (int tn = 0; tn < TS::FN - 1; ++tn) {
       // Issue order inside a group: the read of the next WQ fragment follows the first MFMA, the DMA
@@ -338,35 +366,18 @@ struct GemmTile {
       for (int tm = 0; tm < TS::FM; ++tm) {
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
         if (tm == 0) wf_next = load_frag_b(b_tile, tn + 1, fo);
-        // Large tiles (at most one load per MFMA): the loads of a step are spread over ALL groups in front of the barrier,
-        // XQ first, so that the load path sees them at an even rate.
-        constexpr int ND = TS::LA + TS::LB, GD = TS::FN - 1;
-        const int first = (tn * ND + GD - 1) / GD, next = ((tn + 1) * ND + GD - 1) / GD;   // group tn issues loads [first, next)
-        const int ds = tm - (TS::FM - (next - first));
-        if (PER_SLOT == 1 && ND <= GD * TS::FM) {
-          if (ds >= 0) {
-            const int q = first + ds;
-            if (q < TS::LA) {
-              if constexpr (DMA_A) issue_a(a_dst, k_a, q);
-            } else {
-              if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
-            }
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          continue;
-        }
-        const int d = tm - (TS::FM - SLOTS);
-        if (tn < HALF && d >= 0) {
+        if constexpr (SPREAD) {
+          // Large tiles (at most one load per MFMA): the loads of a step are spread over ALL groups in front of the
+          // barrier, so that the load path sees them at an even rate.
+          const int first = (tn * ND + GD - 1) / GD, next = ((tn + 1) * ND + GD - 1) / GD;   // group tn issues loads [first, next)
+          const int ds = tm - (TS::FM - (next - first));
+          if (ds >= 0) issue(first + ds);
+        } else {
+          const int d = tm - (TS::FM - SLOTS);
+          if (tn < HALF && d >= 0) {
 #pragma unroll
-          for (int j = 0; j < PER_SLOT; ++j) {
-            const int q = tn * NDMA + d * PER_SLOT + j;   // all XQ loads are older than all WQ loads of the step
-            if (d * PER_SLOT + j < NDMA) {
-              if (q < TS::LA) {
-                if constexpr (DMA_A) issue_a(a_dst, k_a, q);
-              } else {
-                if constexpr (DMA_B) issue_b(b_far, k_b, q - TS::LA);
-              }
-            }
+            for (int j = 0; j < PER_SLOT; ++j)
+              if (d * PER_SLOT + j < NDMA) issue(tn * NDMA + d * PER_SLOT + j);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -378,10 +389,10 @@ struct GemmTile {
   }
 
   // The rest of the step: the barrier (NEXT), then the last n fragment, whose XQ fragments are replaced by those of the
-  // next step as they retire.
-  template <bool NEXT, int PENDING>
+  // next step as they retire; A_TAIL: the XQ tile at byte k_a goes into `a_free`, one load behind each MFMA.
+  template <bool NEXT, int PENDING, int NA_TAIL = 0>
   MSLK_AMD_DEVINL void step_tail(const char* a_nxt, const char* b_nxt, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0,
-                                 const v8i& wf_last) {
+                                 const v8i& wf_last, char* a_free = nullptr, int k_a = 0) {
     const FragOff fo = frag_off();
     if constexpr (NEXT) {
       wait_and_barrier<PENDING>();
@@ -391,6 +402,10 @@ struct GemmTile {
 #pragma unroll
     for (int tm = 0; tm < TS::FM; ++tm) {
       acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf_last, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+      if constexpr (NA_TAIL > 0) {   // the first NA_TAIL loads of the XQ tile, spread over the MFMAs
+#pragma unroll
+        for (int q = (tm * NA_TAIL + TS::FM - 1) / TS::FM; q < ((tm + 1) * NA_TAIL + TS::FM - 1) / TS::FM; ++q) issue_a(a_free, k_a, q);
+      }
       if constexpr (NEXT) {
         xf[tm] = load_frag_a<false>(a_next, tm, fo);
         __builtin_amdgcn_sched_barrier(0);  // keep the re-load right behind its MFMA
@@ -400,12 +415,12 @@ struct GemmTile {
   }
 
   // One K step of a ragged tile: as step(), but every n fragment multiplies only the first FMV m fragments of the wave,
-  // the XQ loads of the next step follow the first MFMA group as one block (left out by waves whose rows are all
-  // beyond the valid ones) and the WQ loads follow the second.  Such a step is short: it waits for memory rather than
-  // for the matrix cores, so the fine interleave of step() would buy nothing.
-  template <bool DMA_A, bool DMA_B, bool NEXT, int PENDING, int FMV>
+  // the WQ loads follow the first MFMA group as one block and the XQ loads (left out by waves whose rows are all beyond
+  // the valid ones) the first MFMA behind the barrier.  Such a step is short: it waits for memory rather than for the
+  // matrix cores, so the fine interleave of step() would buy nothing.
+  template <int NA_HEAD, bool DMA_B, bool NEXT, int PENDING, int FMV, int NA_TAIL>
   MSLK_AMD_DEVINL void step_rows(const char* b_cur, char* a_dst, const char* a_nxt, const char* b_nxt, char* b_far, int k_a,
-                                 int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0) {
+                                 int k_b, v4f (&acc)[TS::FN][TS::FM], v8i (&xf)[TS::FM], v8i& wf0, char* a_tail_dst, int k_a_tail) {
     static_assert(TS::FN >= 3 && FMV >= 1 && FMV < TS::FM, "ragged step");
     const FragOff fo = frag_off();
     const char* b_tile = b_tile_of(b_cur);
@@ -417,9 +432,7 @@ struct GemmTile {
       for (int tm = 0; tm < FMV; ++tm)
         acc[tn][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[tn][tm], 0, 0, 0, 0, 0, 0);
       if (tn == 0) {
-        if constexpr (DMA_A) issue_a_live(a_dst, k_a);   // all XQ loads are older than all WQ loads of the step
-      }
-      if (tn == 1) {
+        if constexpr (NA_HEAD > 0) issue_a_live(a_dst, k_a, TS::LA - NA_HEAD, TS::LA);   // older than the WQ loads of the step
         if constexpr (DMA_B) issue_b_all(b_far, k_b);
       }
       wf = wf_next;
@@ -433,6 +446,9 @@ struct GemmTile {
 #pragma unroll
     for (int tm = 0; tm < FMV; ++tm) {
       acc[TS::FN - 1][tm] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wf, xf[tm], acc[TS::FN - 1][tm], 0, 0, 0, 0, 0, 0);
+      if constexpr (NA_TAIL > 0) {
+        if (tm == 0) issue_a_live(a_tail_dst, k_a_tail, 0, NA_TAIL);
+      }
       if constexpr (NEXT) {
         xf[tm] = load_frag_a<true>(a_next, tm, fo);
         __builtin_amdgcn_sched_barrier(0);
@@ -568,14 +584,26 @@ struct GemmTile {
         if (KT > 1 && !DRAIN) wait_and_barrier<TS::LB>();
         else wait_and_barrier<0>();
         load_first_frags<FMV>(a_cur, b_cur, xf, wf0);
-        // step kt multiplies (a_cur, b_cur), fetches XQ of step kt + 1 into a_nxt and WQ of step kt + 2 into b_far
+        // The prologue fetched XQ 0, WQ 0, WQ 1.  Step kt multiplies (the fragments of a_cur, b_cur) and fetches WQ of step
+        // kt + 2 into b_far.  Of every XQ tile the first XT loads are issued two steps ahead (step kt: those of step kt + 2,
+        // behind its barrier, into a_cur), the others one step ahead (step kt: those of step kt + 1, with the WQ loads, into
+        // a_nxt).  Order of issue as a wave sees it: ... XQ(kt+1)[0,XT) | XQ(kt+1)[XT,LA) WQ(kt+2) | barrier kt | XQ(kt+2)[0,XT) ...:
+        // at barrier kt only the LB loads of WQ(kt+2) may be pending.
+        constexpr int XT = XQ_EARLY, XH = TS::LA - XT;
+        if (KT > 1) {
+          if constexpr (FMV < TS::FM) issue_a_live(a_nxt, kBK, 0, XT);
+          else {
+#pragma unroll
+            for (int i = 0; i < XT; ++i) issue_a(a_nxt, kBK, i);
+          }
+        }
         for (int kt = 0; kt < KT - 2; ++kt) {
-          step<true, true, true, TS::LB, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0);
+          step<XH, true, true, TS::LB, FMV, XT>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (kt + 1) * kBK, (kt + 2) * kBK, acc, xf, wf0, a_cur, (kt + 2) * kBK);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
         if (KT > 1) {
-          step<true, false, true, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
+          step<XH, false, true, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, (KT - 1) * kBK, 0, acc, xf, wf0);
           { char* t = a_cur; a_cur = a_nxt; a_nxt = t; }
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
@@ -588,7 +616,7 @@ struct GemmTile {
           last->b_free1 = b_far;
           return;
         }
-        step<false, false, false, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
+        step<0, false, false, 0, FMV>(b_cur, a_nxt, a_nxt, b_nxt, b_far, 0, 0, acc, xf, wf0);
       }
     } else {
       // Symmetric ring: buffer i % RING holds step i; step kt fetches step kt + RING - 1 into the buffers step
@@ -614,16 +642,16 @@ struct GemmTile {
         int kt = 0;
         for (; kt + NS - 1 < KT; ++kt) {
           const int nxt = cur + 1 == NS ? 0 : cur + 1, far = cur == 0 ? NS - 1 : cur - 1;
-          step<true, true, true, (NS - 2) * PER_STEP>(bbuf(cur), abuf(far), abuf(nxt), bbuf(nxt), bbuf(far),
+          step<TS::LA, true, true, (NS - 2) * PER_STEP>(bbuf(cur), abuf(far), abuf(nxt), bbuf(nxt), bbuf(far),
                                                        (kt + NS - 1) * kBK, (kt + NS - 1) * kBK, acc, xf, wf0);
           cur = nxt;
         }
         for (; kt + 1 < KT; ++kt) {   // nothing left to fetch: the first of these steps waits for all that is in flight
           const int nxt = cur + 1 == NS ? 0 : cur + 1;
-          step<false, false, true, 0>(bbuf(cur), abuf(nxt), abuf(nxt), bbuf(nxt), bbuf(nxt), 0, 0, acc, xf, wf0);
+          step<0, false, true, 0>(bbuf(cur), abuf(nxt), abuf(nxt), bbuf(nxt), bbuf(nxt), 0, 0, acc, xf, wf0);
           cur = nxt;
         }
-        step<false, false, false, 0>(bbuf(cur), abuf(cur), abuf(cur), bbuf(cur), bbuf(cur), 0, 0, acc, xf, wf0);
+        step<0, false, false, 0>(bbuf(cur), abuf(cur), abuf(cur), bbuf(cur), bbuf(cur), 0, 0, acc, xf, wf0);
       }
     }
     if (k_tail > 0) {
@@ -632,7 +660,7 @@ struct GemmTile {
       wait_vmcnt0();    // the DMA loads are not visible to the compiler: the wait is explicit
       __syncthreads();
       load_first_frags<FMV>(a_tail, b_tail, xf, wf0);
-      step<false, false, false, 0, FMV>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
+      step<0, false, false, 0, FMV>(b_tail, a_tail, a_tail, b_tail, b_tail, 0, 0, acc, xf, wf0);
     }
     __syncthreads();  // the stages are dead from here on: the epilogue reuses LDS as a transpose buffer
   }
