@@ -130,9 +130,19 @@ def _graph_ms(fn, iters, repeats=5):
     with torch.cuda.graph(graph):
         for i in range(iters):
             fn(i)
-    for _ in range(3):
-        graph.replay()
-    torch.cuda.synchronize()
+    # Capture is host work during which the GPU idles and its clocks fall; a replay of a short graph lasts about a
+    # millisecond, so a few warm-up replays do not bring them back (decode GEMMs measured 0.5 - 2 us per node slower that
+    # way than the same kernels launched one by one after a settling phase).  Replay for the same settling time instead.
+    warm = torch.cuda.Event(enable_timing=True)
+    warm.record()
+    while True:
+        for _ in range(3):
+            graph.replay()
+        now = torch.cuda.Event(enable_timing=True)
+        now.record()
+        now.synchronize()
+        if warm.elapsed_time(now) >= 20.0:
+            break
     times = []
     for _ in range(repeats):
         start = torch.cuda.Event(enable_timing=True)
