@@ -720,7 +720,19 @@ def main():
             api.check(L.mslk_amd_f8f8bf16_rowwise_grouped_stacked(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
                                                                   one.data_ptr(), 1, 8192, 8192, 5120, y4.data_ptr(), api.stream))
 
+        # cfg4's sizes come sorted (largest expert first), the worst order for the equal-count XCD slices of the
+        # device-extent layouts: the same sizes in a fixed shuffled order, as a router would produce them
+        import random
+        shuffled = list(wl4.counts)
+        random.Random(1).shuffle(shuffled)
+        sizes_shuffled = torch.tensor(shuffled, dtype=torch.int64, device=dev)
+
+        def stacked_shuffled_call():
+            api.check(L.mslk_amd_f8f8bf16_rowwise_grouped_stacked(xq4.data_ptr(), WQ4.data_ptr(), xs4.data_ptr(), WS4.data_ptr(),
+                                                                  sizes_shuffled.data_ptr(), 16, 8192, 8192, 5120, y4.data_ptr(), api.stream))
+
         for name, call in (("grouped_stacked_cfg4", stacked_call), ("grouped_mm_2d3d_cfg4", offsets_call),
+                           ("grouped_stacked_cfg4_sizes_shuffled", stacked_shuffled_call),
                            ("batched_16x512x8192x5120", batched_call), ("grouped_one_warm_group_8192x8192x5120", single_group_call)):
             _settle(lambda i: call(), 20.0)
             ms = _median_events_ms(lambda i: call(), 10)
