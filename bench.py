@@ -333,7 +333,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", default="",
-                    help="helper: run only this piece (gemm|gemm-timed|power|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|ceilings) and exit")
+                    help="helper: run only this piece (gemm|gemm-timed|power|phases|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|ceilings) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -371,6 +371,41 @@ def main():
         api.gemm(xq, wq, xs, ws, y)
 
     flops = 2.0 * M * N * K
+    if args.only == "phases":
+        # Where the time of the headline launch goes: the measuring build of the same kernel (four counter readings per
+        # wave, mslk_amd_debug_gemm_phases) on the same operand rotation, on the cfg1 codes and on all-zero codes.
+        stamps = torch.zeros(256 * 4 * 4, dtype=torch.int64, device=dev)
+        out = {}
+        for label in ("cfg1_codes", "zero_codes"):
+            psets = sets if label == "cfg1_codes" else [(torch.zeros_like(xq0), torch.zeros_like(wq0), xs0, ws0, sets[j][4]) for j in range(NSETS)]
+
+            def phase_step(i):
+                xq, wq, xs, ws, y = psets[i % NSETS]
+                api.check(api.L.mslk_amd_debug_gemm_phases(xq.data_ptr(), wq.data_ptr(), xs.data_ptr(), ws.data_ptr(), y.data_ptr(),
+                                                           M, N, K, stamps.data_ptr(), api.stream))
+
+            _settle(phase_step)
+            period_ms = _median_events_ms(phase_step, 200)
+            torch.cuda.synchronize()
+            t = stamps.view(256, 4, 4).cpu().double() * 1e-2   # 100 MHz counter -> microseconds
+            t = t - t[..., 0].min()
+            entry, first, k_end, end = (t[..., i].flatten() for i in range(4))
+
+            def mmm(v):
+                return {"min": round(float(v.min()), 2), "median": round(float(v.median()), 2), "max": round(float(v.max()), 2)}
+
+            xcd_last = [round(float(t[torch.arange(256) % 8 == c][..., 3].max()), 2) for c in range(8)]
+            out[label] = {"us_per_launch_events": round(period_ms * 1e3, 2),
+                          "wave_entry_after_first_entry_us": mmm(entry),
+                          "entry_to_first_operands_us": mmm(first - entry),
+                          "k_loop_31_steps_us": mmm(k_end - first),
+                          "k_loop_per_step_us": mmm((k_end - first) / (K // 128 - 1)),
+                          "last_step_fused_with_epilogue_us": mmm(end - k_end),
+                          "wave_end_after_first_entry_us": mmm(end),
+                          "last_wave_end_per_xcd_us": xcd_last,
+                          "launch_period_minus_last_wave_end_us": round(period_ms * 1e3 - float(end.max()), 2)}
+        print(json.dumps({"gemm_phases_4096": out}))
+        return
     if args.only == "traffic":
         # Counter calibration for `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`: a plain device copy of known
         # size (256 MiB read + 256 MiB written by one elementwise kernel) next to a few GEMM launches.

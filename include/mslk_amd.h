@@ -319,6 +319,19 @@ const char* mslk_amd_debug_dispatch_name(int64_t M, int64_t N, int64_t K, int bi
 int mslk_amd_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, void* stream);
 int mslk_amd_debug_mfma_loop(const void* operands, int form, int iters, int workgroups, void* sink, void* stream);
 
+/*
+ * Where the time of one dense launch goes: the 256 x 256 tile kernel of mslk_amd_f8f8bf16_rowwise (one tile per
+ * workgroup, last K step fused with the epilogue, bf16 output, no bias) built with four readings of the GPU's
+ * constant-rate counter (100 MHz) per wave.  stamps[((workgroup * 4) + wave) * 4 + i], i = 0 kernel entry, 1 first
+ * operands behind the first barrier, 2 the K loop hands its last step to the epilogue, 3 end of the epilogue (the wave's
+ * stores may still be in flight).  Workgroup ids beyond the tile count (the grid is rounded up to a multiple of 8) write
+ * nothing.  M, N multiples of 256, K a multiple of 128 and at least 256: every tile takes the interior path.  Y receives
+ * the product.  `stamps` holds ceil(M/256 * N/256 / 8) * 8 * 16 values.  Not part of the product path; no counterpart in
+ * the reference.
+ */
+int mslk_amd_debug_gemm_phases(const void* xq, const void* wq, const float* x_scale, const float* w_scale, void* y, int64_t M,
+                               int64_t N, int64_t K, uint64_t* stamps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -452,4 +452,18 @@ int mslk_amd_debug_mfma_loop(const void* operands, int form, int iters, int work
   return check_hip(launch_debug_mfma_loop(operands, form, iters, workgroups, sink, (hipStream_t)stream), "mfma loop launch");
 }
 
+int mslk_amd_debug_gemm_phases(const void* xq, const void* wq, const float* x_scale, const float* w_scale, void* y, int64_t M,
+                               int64_t N, int64_t K, uint64_t* stamps, void* stream) {
+  if (M <= 0 || N <= 0 || M % 256 != 0 || N % 256 != 0 || M > (1 << 20) || N > (1 << 20))
+    return fail("debug_gemm_phases: M and N must be positive multiples of 256 (interior tiles only), got M=%lld N=%lld", (long long)M, (long long)N);
+  if (K < 256 || K % 128 != 0 || K > (1 << 24)) return fail("debug_gemm_phases: K must be a multiple of 128, at least 256, got %lld", (long long)K);
+  if ((M / 256) * (N / 256) > (1 << 20)) return fail("debug_gemm_phases: more than 2^20 tiles");
+  if (!xq || !wq || !x_scale || !w_scale || !y || !stamps) return fail("debug_gemm_phases: null pointer");
+  if (reinterpret_cast<uintptr_t>(xq) % 16 || reinterpret_cast<uintptr_t>(wq) % 16 || reinterpret_cast<uintptr_t>(y) % 16 ||
+      reinterpret_cast<uintptr_t>(w_scale) % 16 || reinterpret_cast<uintptr_t>(stamps) % 8)
+    return fail("debug_gemm_phases: operands, output and w_scale must be 16-byte aligned, stamps 8-byte aligned");
+  GemmProblem p{(const uint8_t*)xq, (const uint8_t*)wq, x_scale, w_scale, nullptr, (uint16_t*)y, (int)M, (int)N, (int)K, 0, 0, 0};
+  return check_hip(launch_debug_gemm_phases(p, stamps, (hipStream_t)stream), "gemm phases launch");
+}
+
 }  // extern "C"

@@ -104,6 +104,31 @@ __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p
            p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K);
 }
 
+// Measuring build of dense_tiled_kernel<TileShape<256, 256>> for shapes made of interior tiles only: the same tile
+// map, K loop and fused epilogue, and per wave four readings of the constant-rate counter (100 MHz): kernel entry,
+// first operands behind the first barrier, the K loop's hand-over of its last step, the end of the fused epilogue.
+__global__ __launch_bounds__(256) void dense_phases_kernel(GemmProblem p, int tiles_m, int tiles_n, uint64_t* __restrict__ stamps) {
+  using TS = TileShape<256, 256>;
+  using Tile = GemmTile<TS, 0, false, false, TS::LA / 2, true>;
+  const uint64_t t_entry = __builtin_amdgcn_s_memrealtime();
+  __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
+  int tm, tn;
+  if (!map_tile(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
+  const int m0 = tm * TS::kBM, n0 = tn * TS::kBN;
+  Tile tile;
+  tile.out_f16 = p.out_f16;
+  tile.run_interior(lds, p.xq + (int64_t)m0 * p.K, p.wq + (int64_t)n0 * p.K, p.xs + m0, p.ws + n0, nullptr,
+                    p.y + (int64_t)m0 * p.N + n0, p.N, p.K);
+  const uint64_t t_end = __builtin_amdgcn_s_memrealtime();
+  if ((threadIdx.x & 63) == 0) {
+    uint64_t* o = stamps + ((int64_t)blockIdx.x * 4 + (threadIdx.x >> 6)) * 4;
+    o[0] = t_entry;
+    o[1] = tile.stamp_first_operands;
+    o[2] = tile.stamp_k_loop_end;
+    o[3] = t_end;
+  }
+}
+
 // More tiles than CUs: one workgroup per CU walks its share of the tile list (XCD x keeps its contiguous slice,
 // its workgroups take the entries round-robin, so at any time an XCD works on neighbouring tiles as it does with
 // one workgroup per tile).  The first DMA loads of the next tile are issued before the epilogue of the current one
@@ -374,6 +399,13 @@ hipError_t launch_pad_rows(const uint8_t* src, uint8_t* dst, int64_t rows, int64
   if (dispatch_probe_record("pad_rows")) return hipSuccess;
   const int64_t want = (chunks + 255) / 256;
   pad_rows_kernel<<<(unsigned)(want > 65536 ? 65536 : want), 256, 0, s>>>(src, dst, chunks, (int)(Kp / 16), (int)K);
+  return hipGetLastError();
+}
+
+hipError_t launch_debug_gemm_phases(const GemmProblem& p, uint64_t* stamps, hipStream_t s) {
+  const int tiles_m = p.M / 256, tiles_n = p.N / 256;
+  const int grid = (tiles_m * tiles_n + kXcds - 1) / kXcds * kXcds;
+  dense_phases_kernel<<<(unsigned)grid, 256, 0, s>>>(p, tiles_m, tiles_n, stamps);
   return hipGetLastError();
 }
 

@@ -131,12 +131,16 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* base, uint32_t off, char* lds_wave_bas
 // lane (i, g) the k bytes [16 g, 16 g + 16) and [64 + 16 g, 64 + 16 g + 16) of row i.
 // XQ_EARLY: how many of the LA loads of an XQ tile are issued two K steps ahead instead of one (two-plus-three buffers;
 // see step()).
-template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false, int XQ_EARLY = TS::LA / 2>
+// STAMPS: the wave notes the constant-rate counter (s_memrealtime, 100 MHz) when its first operands are behind the first
+// barrier and when the K loop hands the last step to the fused epilogue -- the measuring build of the dense kernel
+// (mslk_amd_debug_gemm_phases) writes them out beside its own entry and exit times; no other kernel carries them.
+template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false, int XQ_EARLY = TS::LA / 2, bool STAMPS = false>
 struct GemmTile {
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
   uint32_t b_off[TS::LB];
   int out_f16 = 0;          // output element type: 0 bf16, 1 fp16 (set by the caller before run())
+  uint64_t stamp_first_operands = 0, stamp_k_loop_end = 0;   // STAMPS only
   int a_rows = TS::kBM;     // valid rows of the XQ tile (wave-uniform)
   const uint8_t* a_base;    // XQ + m0 * K   (wave-uniform)
   const uint8_t* b_base;    // WQ + n0 * K
@@ -583,6 +587,7 @@ struct GemmTile {
       if (KT > 0) {
         if (KT > 1 && !DRAIN) wait_and_barrier<TS::LB>();
         else wait_and_barrier<0>();
+        if constexpr (STAMPS) stamp_first_operands = __builtin_amdgcn_s_memrealtime();
         load_first_frags<FMV>(a_cur, b_cur, xf, wf0);
         // The prologue fetched XQ 0, WQ 0, WQ 1.  Step kt multiplies (the fragments of a_cur, b_cur) and fetches WQ of step
         // kt + 2 into b_far.  Of every XQ tile the first XT loads are issued two steps ahead (step kt: those of step kt + 2,
@@ -608,6 +613,7 @@ struct GemmTile {
           { char* t = b_cur; b_cur = b_nxt; b_nxt = b_far; b_far = t; }
         }
         if constexpr (HOLD_LAST) {
+          if constexpr (STAMPS) stamp_k_loop_end = __builtin_amdgcn_s_memrealtime();
 #pragma unroll
           for (int tm = 0; tm < TS::FM; ++tm) last->xf[tm] = xf[tm];
           last->wf0 = wf0;

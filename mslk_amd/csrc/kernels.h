@@ -61,6 +61,9 @@ struct GemmProblem {
   int out_f16;        // 0: Y is bf16, 1: Y is fp16
   int w_preshuffled;  // 1: WQ is in the blocked layout [N/16][K/64][4][16][16 B] (N % 16 == 0, K % 64 == 0)
 };
+// The 256 x 256 tile kernel with four counter readings per wave (mslk_amd_debug_gemm_phases): M, N multiples of 256,
+// K a multiple of 128 and at least 256, no bias, bf16 output.
+hipError_t launch_debug_gemm_phases(const GemmProblem& p, uint64_t* stamps, hipStream_t s);
 
 // Dry run of the shape dispatch (mslk_amd_debug_dispatch_name): between dispatch_probe_begin() and dispatch_probe_end()
 // on the calling thread every GEMM launcher records the kernel it would launch (name, tile shape, grid) and launches

@@ -98,6 +98,41 @@ def test_exact_on_full_256_tiles(M, N, K, bias_dtype, fp16_out):
     assert torch.equal(y.cpu(), want.half() if fp16_out else want.bfloat16())
 
 
+def test_measuring_build_of_the_tile_kernel_gives_the_product_bits_and_ordered_stamps():
+    """mslk_amd_debug_gemm_phases is the 256 x 256 tile kernel with four counter readings per wave: it must write the very
+    output of f8f8bf16_rowwise (exact integer arithmetic here), and every wave's readings must be in order."""
+    import ctypes
+    from mslk_amd import _lib
+    M, N, K = 1024, 1280, 512
+    g = torch.Generator().manual_seed(11)
+    xi = torch.randint(-8, 9, (M, K), generator=g).float()
+    wi = torch.randint(-8, 9, (N, K), generator=g).float()
+    xs = 2.0 ** torch.randint(-3, 4, (M,), generator=g).float()
+    ws = 2.0 ** torch.randint(-3, 4, (N,), generator=g).float()
+    want = ((xi @ wi.T) * xs[:, None] * ws[None, :]).bfloat16()
+    xq, wq, xsd, wsd = _gpu(xi.to(F8), wi.to(F8), xs, ws)
+    tiles = (M // 256) * (N // 256)
+    slots = (tiles + 7) // 8 * 8
+    y = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+    stamps = torch.zeros(slots * 16, dtype=torch.int64, device=DEV)
+    L = _lib.lib()
+    _lib.check(L.mslk_amd_debug_gemm_phases(xq.data_ptr(), wq.data_ptr(), xsd.data_ptr(), wsd.data_ptr(), y.data_ptr(), M, N, K,
+                                            stamps.data_ptr(), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(y.cpu(), want)
+    assert torch.equal(y, torch.ops.mslk.f8f8bf16_rowwise(xq, wq, xsd, wsd))
+    t = stamps.view(slots, 4, 4).cpu()
+    written = t[..., 0] != 0
+    assert int(written.all(dim=1).sum()) == tiles and int(written.any(dim=1).sum()) == tiles   # one workgroup per tile, all four waves
+    w = t[written.all(dim=1)]
+    assert bool((w[..., 0] <= w[..., 1]).all() and (w[..., 1] <= w[..., 2]).all() and (w[..., 2] <= w[..., 3]).all())
+    assert int((w[..., 3] - w[..., 0]).max()) < 100_000   # 100 MHz counter: under a millisecond
+    # shapes with edge tiles are refused: the measuring build has the interior path only
+    assert L.mslk_amd_debug_gemm_phases(xq.data_ptr(), wq.data_ptr(), xsd.data_ptr(), wsd.data_ptr(), y.data_ptr(), M - 1, N, K,
+                                        stamps.data_ptr(), None) != 0
+    assert b"multiples of 256" in L.mslk_amd_last_error()
+
+
 def test_identity_and_one_hot_weights_select_dequantized_activations():
     g = torch.Generator().manual_seed(9)
     M, K = 300, 512
