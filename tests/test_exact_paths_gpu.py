@@ -92,6 +92,28 @@ def test_tensorlist_grouped_exact(ms, N, K):
             _same_bits(ys[e], _want(xi[e], wi[e], xs[e], ws[e]), f"group {e} ({m} rows)")
 
 
+@pytest.mark.parametrize("K", [128, 256, 384])
+def test_tensorlist_grouped_exact_on_k_loops_of_one_two_and_three_steps(K):
+    """The operator refuses K < 512 as the reference does (fp8_rowwise_grouped_gemm.hip:505-507); the C ABI does not, and the
+    start and the end of the software pipeline of the K loop are exactly what such short loops consist of."""
+    import ctypes
+    from mslk_amd import _lib
+    ms, N = [m for m in ROWSKIP_256 if m], 512
+    g = torch.Generator().manual_seed(sum(ms) + N + K)
+    xi, wi, xs, ws = _groups(ms, N, K, g)
+    xq, wq = [t.to(F8).to(DEV) for t in xi], [t.to(F8).to(DEV) for t in wi]
+    xsd, wsd = [t.to(DEV) for t in xs], [t.to(DEV) for t in ws]
+    ys = [torch.full((m, N), SENTINEL, dtype=torch.bfloat16, device=DEV) for m in ms]
+    G = len(ms)
+    P, I = ctypes.c_void_p * G, ctypes.c_int64 * G
+    ptrs = lambda ts: P(*[t.data_ptr() for t in ts])
+    _lib.check(_lib.lib().mslk_amd_f8f8bf16_rowwise_grouped(G, ptrs(xq), ptrs(wq), ptrs(xsd), ptrs(wsd), ptrs(ys), I(*ms), I(*[N] * G),
+                                                            I(*[K] * G), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    for e, m in enumerate(ms):
+        _same_bits(ys[e], _want(xi[e], wi[e], xs[e], ws[e]), f"group {e} ({m} rows)")
+
+
 def _stacked_case(ms, N, K, g, extra=0):
     G, total = len(ms), sum(ms) + extra
     xi, wi = _ints(total, K, g), _ints(G * N, K, g)
@@ -115,6 +137,9 @@ MANY_130 = [((i * 53) % 97 if i % 4 else 0) + (260 if i % 31 == 7 else 0) for i 
     (ROWSKIP_128, 512, 656, 5),                                        # 128 x 128 tiles, every row-skipping class, a K tail
     (MANY_70, 512, 512, 9),                                            # more than 64 groups: a second chunk of extents
     (MANY_130, 520, 528, 0),                                           # more than 128: a third; N % 256 != 0
+    ([1024 + 40, 1024 + 100, 1024 + 180, 1024 + 250], 512, 256, 0),     # 256 x 256 tiles, K loops of two and of three steps
+    ([1024 + 40, 1024 + 100, 1024 + 180, 1024 + 250], 512, 384, 3),
+    (ROWSKIP_128, 512, 256, 0),                                        # the same on 128 x 128 tiles
 ])
 def test_stacked_and_offsets_over_m_exact(ms, N, K, extra):
     """grouped_device_kernel with int64 sizes (stacked) and int32 cumulative ends (2D-3D): the same bits from both, rows
