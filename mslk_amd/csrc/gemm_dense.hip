@@ -80,21 +80,23 @@ MSLK_AMD_DEVINL bool map_tile(int bid, int tiles_m, int tiles_n, int& tm, int& t
   return true;
 }
 
-template <typename TS, int BIAS, bool PS>
+// WS: the weights are fetched with non-temporal loads (shapes of one or two row tiles: no other tile of the XCD asks for
+// a weight line again).
+template <typename TS, int BIAS, bool PS, bool WS = false>
 __global__ __launch_bounds__(TS::NTHREADS) void dense_tiled_kernel(GemmProblem p, int tiles_m, int tiles_n) {
   constexpr int BM = TS::kBM, BN = TS::kBN;
   __shared__ __attribute__((aligned(1024))) char lds[TS::LDS_BYTES];
   int tm, tn;
   if (!map_tile(blockIdx.x, tiles_m, tiles_n, tm, tn)) return;
   const int m0 = tm * BM, n0 = tn * BN;
-  GemmTile<TS, BIAS, PS> tile;
+  GemmTile<TS, BIAS, PS, false, TS::LA / 2, false, WS> tile;
   tile.out_f16 = p.out_f16;
   const void* bias = nullptr;
   if constexpr (BIAS == 1) bias = reinterpret_cast<const float*>(p.bias) + n0;
   if constexpr (BIAS == 2) bias = reinterpret_cast<const uint16_t*>(p.bias) + n0;
   if constexpr (BIAS == 0 && TS::RING == 0 && TS::NW == 4 && TS::FM * TS::FN * 4 >= 256) {
     // tiles with every row and column: the epilogue starts inside the last K step
-    if (GemmTile<TS, BIAS, PS>::interior_ok(p.ws + n0, bias, p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K)) {
+    if (decltype(tile)::interior_ok(p.ws + n0, bias, p.y + (int64_t)m0 * p.N + n0, p.M - m0, p.N - n0, p.N, p.K)) {
       tile.run_interior(lds, p.xq + (int64_t)m0 * p.K, p.wq + (int64_t)n0 * p.K, p.xs + m0, p.ws + n0, bias,
                         p.y + (int64_t)m0 * p.N + n0, p.N, p.K);
       return;
@@ -196,19 +198,36 @@ hipError_t launch_persistent_shape(const GemmProblem& p, int wgs, hipStream_t s)
   return hipGetLastError();
 }
 
-template <typename TS, bool PS>
+// STREAM_W: 0 never; 1 when the shape is one row of tiles, so that every weight line is asked for exactly once (measured at
+// M = 16 ... 128 on six weight shapes: 3 - 11 % faster, e.g. N = K = 8192, M = 16: 14.9 -> 13.3 us; with two row tiles it
+// depends on whether the two land in one XCD at the same time: 9 % faster at N = 28672, 24 % slower at 4096 x 14336);
+// 2 always (tile shapes that are only picked for a single row of tiles).
+template <typename TS, bool PS, int STREAM_W = 0>
 hipError_t launch_tiled_shape(const GemmProblem& p, hipStream_t s) {
   constexpr int BM = TS::kBM, BN = TS::kBN;
   const int tiles_m = (p.M + BM - 1) / BM, tiles_n = (p.N + BN - 1) / BN;
   const int ntiles = tiles_m * tiles_n;
   const int grid = ((ntiles + kXcds - 1) / kXcds) * kXcds;
-  if (dispatch_probe_record("dense_tiled<%d,%d,waves=%dx%d,ring=%d>%s tiles=%d", BM, BN, TS::WM, TS::WN, TS::RING,
-                            PS ? " preshuffled" : "", ntiles))
+  const bool stream = STREAM_W == 2 || (STREAM_W == 1 && tiles_m == 1);
+  if (dispatch_probe_record("dense_tiled<%d,%d,waves=%dx%d,ring=%d>%s%s tiles=%d", BM, BN, TS::WM, TS::WN, TS::RING,
+                            PS ? " preshuffled" : "", stream ? " weights streamed" : "", ntiles))
     return hipSuccess;
-  switch (p.bias_dtype) {
-    case 0: dense_tiled_kernel<TS, 0, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
-    case 1: dense_tiled_kernel<TS, 1, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
-    default: dense_tiled_kernel<TS, 2, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+  if constexpr (STREAM_W != 0) {
+    if (stream || STREAM_W == 2) {
+      switch (p.bias_dtype) {
+        case 0: dense_tiled_kernel<TS, 0, PS, true><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+        case 1: dense_tiled_kernel<TS, 1, PS, true><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+        default: dense_tiled_kernel<TS, 2, PS, true><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+      }
+      return hipGetLastError();
+    }
+  }
+  if constexpr (STREAM_W != 2) {
+    switch (p.bias_dtype) {
+      case 0: dense_tiled_kernel<TS, 0, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+      case 1: dense_tiled_kernel<TS, 1, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+      default: dense_tiled_kernel<TS, 2, PS><<<grid, TS::NTHREADS, 0, s>>>(p, tiles_m, tiles_n); break;
+    }
   }
   return hipGetLastError();
 }
@@ -341,9 +360,9 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // hold two move twice the activation bytes; 64 x 64 tiles halve the tile count and the activation traffic
   // (N = 10240, K = 8192, M = 64: 33.3 -> 28.3 us; N = 57344, K = 4096, M = 64: 68.4 -> 55.5 us).
   if (p.M <= 64 && p.N >= kShortTileMinN) {
-    if (p.M <= 32 && p.N <= 16384) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false>(p, s);
-    if (p.M <= 32 || p.N <= 8192) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false>(p, s);
-    return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false>(p, s);
+    if (p.M <= 32 && p.N <= 16384) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false, 2>(p, s);
+    if (p.M <= 32 || p.N <= 8192) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false, 2>(p, s);
+    return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false, 1>(p, s);
   }
   if (big_tiles > cus) return launch_persistent_shape<TileShape<256, 256>, false>(p, cus, s);
   // 128 x 256 tiles (wave tile 64 x 128, three ring buffers, one workgroup per CU) when they cover 160 ... 256 CUs in
@@ -355,12 +374,12 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
     const int64_t rows128 = (p.M + 127) / 128;
     const int64_t tiles12 = rows128 * ((p.N + 255) / 256);
     if (tiles12 >= cus * 5 / 8 && tiles12 <= cus && (big_tiles < cus * 5 / 8 || rows128 % 2 == 1))
-      return launch_tiled_shape<TileShape<128, 256, 2, 2, 3>, false>(p, s);
+      return launch_tiled_shape<TileShape<128, 256, 2, 2, 3>, false, 1>(p, s);
   }
   // Otherwise 256 x 256 tiles from 129 tiles on: the 128 x 256 tiles would then need two passes and the co-resident
   // 128 x 128 tiles more than two per CU (N = 6144, M = 1536: 144 tiles, K = 8192: 100.0 -> 87.1 us, K = 4096:
   // 48.9 -> 39.5 us).
-  if (big_tiles > cus / 2) return launch_tiled_shape<TileShape<256, 256>, false>(p, s);
+  if (big_tiles > cus / 2) return launch_tiled_shape<TileShape<256, 256>, false, 1>(p, s);
   // M > 64 with at most one 64 x 64 tile per CU: such tiles (four waves stacked along M, five ring buffers, two
   // workgroups per CU) wherever they cover at least as many CUs as the 128-row tiles below would, in a single pass:
   // rows 65 ... 128 then do not cost a second, half-empty 128-row tile's worth of activation traffic (N = K = 8192,
@@ -369,11 +388,11 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
     const int64_t tiles64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
     const int64_t rows128 = (p.M + 127) / 128;
     const int64_t tiles128 = small_tiles <= cus / 4 ? rows128 * ((p.N + 31) / 32) : small_tiles <= cus / 2 ? rows128 * ((p.N + 63) / 64) : small_tiles;
-    if (tiles64 <= cus && tiles64 >= tiles128) return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false>(p, s);
+    if (tiles64 <= cus && tiles64 >= tiles128) return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false, 1>(p, s);
   }
-  if (small_tiles <= cus / 4 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false>(p, s);
-  if (small_tiles <= cus / 2 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false>(p, s);
-  if (small_tiles <= cus) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false>(p, s);
+  if (small_tiles <= cus / 4 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false, 1>(p, s);
+  if (small_tiles <= cus / 2 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false, 1>(p, s);
+  if (small_tiles <= cus) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false, 1>(p, s);
   return launch_tiled_shape<TileShape<128, 128>, false>(p, s);
 }
 

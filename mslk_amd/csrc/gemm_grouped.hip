@@ -48,9 +48,17 @@ __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
   int tm, tn;
   local_tile(t - d.tile_begin, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  GemmTile<TS, 0, false, true> tile;   // ROWSKIP: the ragged last row tile of a group costs what its rows cost
-  tile.run(lds, d.xq + (int64_t)m0 * d.K, d.wq + (int64_t)n0 * d.K, d.xs + m0, d.ws + n0, nullptr,
-           d.y + (int64_t)m0 * d.N + n0, d.M - m0, d.N - n0, d.N, d.K);
+  // ROWSKIP: the ragged last row tile of a group costs what its rows cost.  A group of a single row tile is the only
+  // reader of its weight block: its tiles fetch the weights with non-temporal loads.
+  if (tiles_m == 1) {
+    GemmTile<TS, 0, false, true, TS::LA / 2, false, true> tile;
+    tile.run(lds, d.xq + (int64_t)m0 * d.K, d.wq + (int64_t)n0 * d.K, d.xs + m0, d.ws + n0, nullptr,
+             d.y + (int64_t)m0 * d.N + n0, d.M - m0, d.N - n0, d.N, d.K);
+  } else {
+    GemmTile<TS, 0, false, true> tile;
+    tile.run(lds, d.xq + (int64_t)m0 * d.K, d.wq + (int64_t)n0 * d.K, d.xs + m0, d.ws + n0, nullptr,
+             d.y + (int64_t)m0 * d.N + n0, d.M - m0, d.N - n0, d.N, d.K);
+  }
 }
 
 // Groups whose extents live in device memory (or are uniform).  `layout` says which dimension varies
@@ -275,8 +283,17 @@ __global__ __launch_bounds__(256) void grouped_device_kernel(DeviceGroups p) {
     slow_tile<BM, BN, BIAS>(a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, K);
     return;
   }
-  GemmTile<TS, BIAS, false, true> tile;
-  tile.run(lds, a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, (uint32_t)p.K);
+  // A weight block that a single row tile reads (a group of at most BM rows, or every group of a batch of such) is
+  // fetched with non-temporal loads (cfg4 307 -> 298 us, four big experts + eight of 256 rows 276 -> 253 us; with groups
+  // of two row tiles included: cfg4 304 -> 315 us, a uniform batch of 512-row groups 268 -> 263 us -- not taken).
+  const int row_tiles = ((LAYOUT == kGroupsPrepadM ? p.M : Mg) + BM - 1) / BM;
+  if (row_tiles == 1) {
+    GemmTile<TS, BIAS, false, true, TS::LA / 2, false, true> tile;
+    tile.run(lds, a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, (uint32_t)p.K);
+  } else {
+    GemmTile<TS, BIAS, false, true> tile;
+    tile.run(lds, a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, (uint32_t)p.K);
+  }
 }
 
 template <int LAYOUT, int BM, int BN, int BIAS>

@@ -118,9 +118,15 @@ MSLK_AMD_DEVINL const uint8_t* uniform_ptr(const uint8_t* p) {
   const uint32_t lo = __builtin_amdgcn_readfirstlane((int)(uint32_t)v), hi = __builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
   return reinterpret_cast<const uint8_t*>(((uint64_t)hi << 32) | lo);
 }
+// STREAM: the bytes are read once by this launch (a weight tile that no other row tile of its XCD shares): the load is
+// marked non-temporal, so the line does not displace what the L2 is asked for again.
+template <bool STREAM = false>
 MSLK_AMD_DEVINL void dma16(const uint8_t* base, uint32_t off, char* lds_wave_base) {
   const uint32_t dst = (uint32_t)(uintptr_t)(lds_ptr_t)lds_wave_base;
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(dst) : "memory", "m0");
+  if constexpr (STREAM)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 nt" : : "v"(off), "s"(base), "s"(dst) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(dst) : "memory", "m0");
 }
 
 
@@ -134,7 +140,10 @@ MSLK_AMD_DEVINL void dma16(const uint8_t* base, uint32_t off, char* lds_wave_bas
 // STAMPS: the wave notes the constant-rate counter (s_memrealtime, 100 MHz) when its first operands are behind the first
 // barrier and when the K loop hands the last step to the fused epilogue -- the measuring build of the dense kernel
 // (mslk_amd_debug_gemm_phases) writes them out beside its own entry and exit times; no other kernel carries them.
-template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false, int XQ_EARLY = TS::LA / 2, bool STAMPS = false>
+// W_STREAM: the weight tile is fetched with non-temporal loads (dma16<true>): for tiles whose weight block at most two row
+// tiles share.
+template <typename TS, int BIAS, bool PS = false, bool ROWSKIP = false, int XQ_EARLY = TS::LA / 2, bool STAMPS = false,
+          bool W_STREAM = false>
 struct GemmTile {
   // Per-lane state that is constant over the K loop.
   uint32_t a_off[TS::LA];   // byte offset of this lane's 16-byte chunk relative to a_base, k = 0
@@ -189,7 +198,7 @@ struct GemmTile {
   }
   MSLK_AMD_DEVINL void issue_b(char* bbuf, int k0, int i) {
     // pre-shuffled: the K step at byte k0 starts 16 rows x k0 bytes into the row group
-    dma16(b_base + (PS ? k0 * 16 : k0), b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
+    dma16<W_STREAM>(b_base + (PS ? k0 * 16 : k0), b_off[i], bbuf + (wave_id() * TS::LB + i) * 1024);
   }
   MSLK_AMD_DEVINL void issue_a_all(char* abuf, int k0) {
 #pragma unroll
@@ -227,7 +236,7 @@ struct GemmTile {
       const int chunk = (lane & 7) ^ lds_swz(row);
       char* dst = bbuf + (wave * TS::LB + i) * 1024;
       const bool valid = PS ? ((wave * TS::LB + i) & 1) * 64 < k_valid : chunk * 16 < k_valid;
-      if (valid) dma16(b_base + (PS ? k0 * 16 : k0), b_off[i], dst);
+      if (valid) dma16<W_STREAM>(b_base + (PS ? k0 * 16 : k0), b_off[i], dst);
       else *reinterpret_cast<uint4*>(dst + lane * 16) = make_uint4(0, 0, 0, 0);
     }
   }

@@ -155,13 +155,13 @@ DISPATCH_TABLE = [
     ((8192, 28672, 4096, 2, 0, 0, 1), "dense_persistent<256,256> tiles=3584 workgroups=256"),                # cfg2
     ((1, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),                 # cfg3, M = 1
     ((4, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),
-    ((16, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> tiles=256"),
-    ((64, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,32,waves=4x1,ring=6> tiles=256"),
+    ((16, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> weights streamed tiles=256"),
+    ((64, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,32,waves=4x1,ring=6> weights streamed tiles=256"),
     ((16, 8192, 8192, 0, 0, 1, 1), "skinny_lds<m_frags=1,n_frags=2,steps=2> preshuffled workgroups=256"),    # cfg3 on blocked weights
     ((64, 8192, 8192, 0, 0, 1, 1), "skinny_lds<m_frags=4,n_frags=2,steps=1> preshuffled workgroups=256"),
     ((64, 4096, 14336, 0, 0, 0, 1), "skinny_lds<m_frags=4,n_frags=1,steps=1> workgroups=256"),
     ((8, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),                  # last M of the streaming kernel on wide weights
-    ((9, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> tiles=256"),
+    ((9, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> weights streamed tiles=256"),
     ((3, 1000, 272, 0, 0, 0, 1), "skinny_registers<m_frags=1,n_frags=1,steps=8> workgroups=63"),              # K % 1024 != 0
     ((8192, 8192, 8192, 0, 0, 0, 1), "dense_persistent<256,256> tiles=1024 workgroups=256"),
     ((2304, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256 + dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
@@ -170,6 +170,9 @@ DISPATCH_TABLE = [
     ((512, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,128,waves=2x2,ring=5> tiles=256"),
     ((256, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
     ((128, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=256"),
+    ((64, 10240, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> weights streamed tiles=160"),         # one row of tiles: non-temporal weight loads
+    ((128, 28672, 4096, 0, 0, 0, 1), "dense_tiled<128,128,waves=2x2,ring=5> weights streamed tiles=224"),
+    ((100, 57344, 8192, 0, 0, 0, 1), "dense_tiled<128,256,waves=2x2,ring=3> weights streamed tiles=224"),
     ((4096, 8192, 4096, 0, 0, 0, 1), "dense_persistent<256,256> tiles=512 workgroups=256"),
     ((4096, 4096, 4096, 0, 1, 1, 1), "dense_tiled<256,256,waves=2x2,ring=0> preshuffled tiles=256"),
     ((4096, 4096, 4100, 0, 0, 0, 1), "pad_rows + pad_rows + dense_tiled<256,256,waves=2x2,ring=0> tiles=256"),
