@@ -282,7 +282,7 @@ def _ceilings(api):
     # ---- streaming read: six distinct 64 MiB buffers (more than the 256 MB Infinity Cache) and one 1 GiB buffer
     small = [torch.randint(0, 255, (64 << 20,), dtype=torch.uint8, device=dev) for _ in range(6)]
     big = torch.randint(0, 255, (1 << 30,), dtype=torch.uint8, device=dev)
-    for mode, mname in ((0, "register_loads"), (1, "lds_dma_loads")):
+    for mode, mname in ((0, "register_loads"), (1, "lds_dma_loads"), (2, "lds_dma_loads_nontemporal")):
         for label, bufs in (("64MiB", small), ("1GiB", [big])):
             best = None
             for wgs in (512, 1024, 2048, 4096):

@@ -310,7 +310,8 @@ const char* mslk_amd_debug_dispatch_name(int64_t M, int64_t N, int64_t K, int bi
  * peak figures, bench/gemm/gemm_bench.py:61-68) and not part of the product path.
  *   mslk_amd_debug_stream_read: `workgroups` x 256 lanes read `bytes` from `src` once and write nothing.  mode 0: 16-byte
  *     non-temporal loads into registers (bytes % 16 == 0); mode 1: the global -> LDS DMA loads the GEMM kernels use
- *     (bytes % 1024 == 0).  `sink` (device int, may be NULL) is never written for real inputs.
+ *     (bytes % 1024 == 0); mode 2: the same with the non-temporal bit, as the kernels fetch weights that are read once.
+ *     `sink` (device int, may be NULL) is never written for real inputs.
  *   mslk_amd_debug_mfma_loop: `workgroups` x 4 waves each run `iters` iterations of a 128 x 128 x 128 wave tile out of
  *     registers: 64 v_mfma_f32_16x16x128_f8f6f4 (form 0) or 32 v_mfma_f32_32x32x64_f8f6f4 (form 1) per iteration, i.e.
  *     iters * 2 * 128^3 FLOP per wave.  `operands` points at 128 KiB of e4m3 codes (32-byte aligned) that fill the operand

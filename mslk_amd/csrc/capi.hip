@@ -436,7 +436,7 @@ const char* mslk_amd_debug_dispatch_name(int64_t M, int64_t N, int64_t K, int bi
 }
 
 int mslk_amd_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, void* stream) {
-  if (mode != 0 && mode != 1) return fail("debug_stream_read: mode must be 0 (register loads) or 1 (LDS DMA loads)");
+  if (mode < 0 || mode > 2) return fail("debug_stream_read: mode must be 0 (register loads), 1 (LDS DMA loads) or 2 (non-temporal LDS DMA loads)");
   if (bytes < 0 || bytes % (mode == 0 ? 16 : 1024) != 0) return fail("debug_stream_read: bytes must be a non-negative multiple of %d", mode == 0 ? 16 : 1024);
   if (workgroups <= 0 || workgroups > 65536) return fail("debug_stream_read: workgroups must be in 1 .. 65536");
   if (bytes == 0) return 0;

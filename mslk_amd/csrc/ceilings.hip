@@ -32,7 +32,9 @@ __global__ __launch_bounds__(256) void stream_read_kernel(const v4i* __restrict_
 }
 
 // The same bytes through the global -> LDS DMA form of the load, the way the GEMM kernels fetch their operands: each
-// wave moves 1 KiB per instruction into a private 16 KiB ring and never reads it back.
+// wave moves 1 KiB per instruction into a private 16 KiB ring and never reads it back.  NT: with the non-temporal bit,
+// as the kernels fetch weights that are read once.
+template <bool NT>
 __global__ __launch_bounds__(256) void stream_dma_kernel(const uint8_t* __restrict__ src, int64_t kib, int* __restrict__ sink) {
   __shared__ __attribute__((aligned(1024))) char lds[4 * 16 * 1024];
   const int lane = threadIdx.x & 63;
@@ -41,7 +43,7 @@ __global__ __launch_bounds__(256) void stream_dma_kernel(const uint8_t* __restri
   const int64_t waves = (int64_t)gridDim.x * 4;
   int slot = 0;
   for (int64_t b = (int64_t)blockIdx.x * 4 + wave; b < kib; b += waves) {
-    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + b * 1024 + lane * 16), (lds_ptr_t)(ring + slot * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gbl_ptr_t)(src + b * 1024 + lane * 16), (lds_ptr_t)(ring + slot * 1024), 16, 0, NT ? 2 : 0);
     slot = (slot + 1) & 15;
   }
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the loads have landed before the wave ends
@@ -114,7 +116,8 @@ __global__ __launch_bounds__(256) void mfma_32x32x64_kernel(const v8i* __restric
 
 hipError_t launch_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, hipStream_t s) {
   if (mode == 0) stream_read_kernel<<<workgroups, 256, 0, s>>>(static_cast<const v4i*>(src), bytes / 16, static_cast<int*>(sink));
-  else stream_dma_kernel<<<workgroups, 256, 0, s>>>(static_cast<const uint8_t*>(src), bytes / 1024, static_cast<int*>(sink));
+  else if (mode == 1) stream_dma_kernel<false><<<workgroups, 256, 0, s>>>(static_cast<const uint8_t*>(src), bytes / 1024, static_cast<int*>(sink));
+  else stream_dma_kernel<true><<<workgroups, 256, 0, s>>>(static_cast<const uint8_t*>(src), bytes / 1024, static_cast<int*>(sink));
   return hipGetLastError();
 }
 

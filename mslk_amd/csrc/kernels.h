@@ -17,8 +17,9 @@ hipError_t launch_dequantize_fp8_row(const void* xq, const float* scale, int64_t
 hipError_t launch_preshuffle_b(const void* src, void* dst, int64_t G, int64_t N, int64_t K, hipStream_t s);
 hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t s);
 // Ceiling probes (ceilings.hip): a pure read of `bytes` from src (mode 0: 16-byte loads into registers, bytes % 16 == 0;
-// mode 1: global -> LDS DMA loads, bytes % 1024 == 0), and a register-only MFMA loop (form 0: 16x16x128, form 1:
-// 32x32x64) of `iters` 128 x 128 x 128 wave tiles per wave on the 128 KiB of operand bytes at `operands`.
+// mode 1: global -> LDS DMA loads, mode 2: the same non-temporal, bytes % 1024 == 0), and a register-only MFMA loop
+// (form 0: 16x16x128, form 1: 32x32x64) of `iters` 128 x 128 x 128 wave tiles per wave on the 128 KiB of operand bytes
+// at `operands`.
 hipError_t launch_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, hipStream_t s);
 hipError_t launch_debug_mfma_loop(const void* operands, int form, int iters, int workgroups, void* sink, hipStream_t s);
 
