@@ -22,13 +22,15 @@ namespace {
 constexpr int kXcds = 8;
 constexpr int kGroupM = 4;
 
-// Tile order inside one group: panels of kGroupM row tiles, column-major inside a panel.
-MSLK_AMD_DEVINL void local_tile(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
+// Tile order inside one group: panels of kGroupM row tiles, column-major inside a panel.  Returns the number of row tiles
+// of the tile's panel: the tiles that read one weight block at about the same time.
+MSLK_AMD_DEVINL int local_tile(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
   const int panel = kGroupM * tiles_n;
   const int first_m = (t / panel) * kGroupM;
   const int rows = tiles_m - first_m < kGroupM ? tiles_m - first_m : kGroupM;
   tm = first_m + (t % panel) % rows;
   tn = (t % panel) / rows;
+  return rows;
 }
 
 template <int BM, int BN>
@@ -46,11 +48,11 @@ __global__ __launch_bounds__(256) void grouped_tiled_kernel(GroupTable tab) {
   const GroupDesc& d = tab.g[gi];
   const int tiles_m = (d.M + BM - 1) / BM, tiles_n = (d.N + BN - 1) / BN;
   int tm, tn;
-  local_tile(t - d.tile_begin, tiles_m, tiles_n, tm, tn);
+  const int panel_rows = local_tile(t - d.tile_begin, tiles_m, tiles_n, tm, tn);
   const int m0 = tm * BM, n0 = tn * BN;
-  // ROWSKIP: the ragged last row tile of a group costs what its rows cost.  A group of a single row tile is the only
-  // reader of its weight block: its tiles fetch the weights with non-temporal loads.
-  if (tiles_m == 1) {
+  // ROWSKIP: the ragged last row tile of a group costs what its rows cost.  A tile alone in its panel is the only reader
+  // of its weight block at that time: it fetches the weights with non-temporal loads.
+  if (panel_rows == 1) {
     GemmTile<TS, 0, false, true, TS::LA / 2, false, true> tile;
     tile.run(lds, d.xq + (int64_t)m0 * d.K, d.wq + (int64_t)n0 * d.K, d.xs + m0, d.ws + n0, nullptr,
              d.y + (int64_t)m0 * d.N + n0, d.M - m0, d.N - n0, d.N, d.K);
@@ -283,11 +285,12 @@ __global__ __launch_bounds__(256) void grouped_device_kernel(DeviceGroups p) {
     slow_tile<BM, BN, BIAS>(a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, K);
     return;
   }
-  // A weight block that a single row tile reads (a group of at most BM rows, or every group of a batch of such) is
-  // fetched with non-temporal loads (cfg4 307 -> 298 us, four big experts + eight of 256 rows 276 -> 253 us; with groups
-  // of two row tiles included: cfg4 304 -> 315 us, a uniform batch of 512-row groups 268 -> 263 us -- not taken).
-  const int row_tiles = ((LAYOUT == kGroupsPrepadM ? p.M : Mg) + BM - 1) / BM;
-  if (row_tiles == 1) {
+  // A weight block that a single row tile reads at a time (the tile is the only one of its panel with rows to compute:
+  // a group of at most BM rows, or the last panel of a group of 4 k + 1 row tiles) is fetched with non-temporal loads
+  // (cfg4 307 -> 298 us, four big experts + eight of 256 rows 276 -> 253 us; with panels of two row tiles included:
+  // cfg4 304 -> 315 us, a uniform batch of 512-row groups 268 -> 263 us -- not taken).
+  const int live_tiles = (Mg + BM - 1) / BM, panel_first = tm / kGroupM * kGroupM;
+  if (live_tiles - panel_first == 1) {
     GemmTile<TS, BIAS, false, true, TS::LA / 2, false, true> tile;
     tile.run(lds, a, b, xs, ws, bias, y, m_rem, n_rem, p.N, Kg, (uint32_t)p.K);
   } else {
