@@ -296,6 +296,32 @@ def _ceilings(api):
             nbytes = bufs[0].numel()
             out[f"stream_read_{mname}_{label}"] = {"ms": best[0], "workgroups": best[1], "TBps": nbytes / (best[0] * 1e-3) / 1e12,
                                                    "frac_of_8TBps": nbytes / (best[0] * 1e-3) / PEAK_HBM_BPS}
+    # ---- the operand streams of a medium-M shape alone: M = 256, N = K = 8192 on 128 x 64 tiles (256 workgroups, two row
+    # tiles), activations from the L2, weights from HBM (the six 64 MiB buffers in turn), without LDS reads or multiplies;
+    # beside them the GEMM itself on the same bytes
+    Mt, Nt, Kt = 256, 8192, 8192
+    xbuf = small[0][: Mt * Kt].clone()
+    ones_m, ones_n = torch.ones(Mt, device=dev), torch.ones(Nt, device=dev)
+    yt = torch.empty(Mt, Nt, dtype=torch.bfloat16, device=dev)
+    for b in small + [xbuf]:
+        b &= 0x77                                            # no NaN codes, so that the GEMM beside the probe multiplies finite values
+    streams = {}
+    for which, wname in ((1, "activations_only"), (2, "weights_only"), (3, "both")):
+        def step(i, which=which):
+            b = small[i % len(small)]
+            api.check(L.mslk_amd_debug_tile_streams(xbuf.data_ptr(), xbuf.numel(), b.data_ptr(), b.numel(), Kt, Mt // 128, Nt // 64,
+                                                    which, api.stream))
+        _settle(step, 10.0)
+        streams[wname + "_us"] = _median_events_ms(step, 60) * 1e3
+    f8 = torch.float8_e4m3fn
+    def gemm_step(i):
+        api.gemm(xbuf.view(f8).view(Mt, Kt), small[i % len(small)].view(f8).view(Nt, Kt), ones_m, ones_n, yt)
+    _settle(gemm_step, 10.0)
+    streams["gemm_us"] = _median_events_ms(gemm_step, 60) * 1e3
+    streams["gemm_kernel"] = L.mslk_amd_debug_dispatch_name(Mt, Nt, Kt, 0, 0, 0, 1).decode()
+    streams["MB_activations_per_launch_from_L2"] = (Mt // 128) * (Nt // 64) * 128 * Kt / 1e6
+    streams["MB_weights_per_launch_from_HBM"] = Nt * Kt / 1e6
+    out["tile_streams_M256_N8192_K8192"] = streams
     del small, big
     # the launch itself: the same kernel on 16 bytes
     tiny = torch.zeros(1024, dtype=torch.uint8, device=dev)

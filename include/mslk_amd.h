@@ -316,9 +316,17 @@ const char* mslk_amd_debug_dispatch_name(int64_t M, int64_t N, int64_t K, int bi
  *     registers: 64 v_mfma_f32_16x16x128_f8f6f4 (form 0) or 32 v_mfma_f32_32x32x64_f8f6f4 (form 1) per iteration, i.e.
  *     iters * 2 * 128^3 FLOP per wave.  `operands` points at 128 KiB of e4m3 codes (32-byte aligned) that fill the operand
  *     registers once; the rate depends on these values through the power they draw.
+ *   mslk_amd_debug_tile_streams: the global -> LDS loads of the 128 x 64 tile kernel's K loop and nothing else (no LDS
+ *     reads, no multiplies, no output): tiles_m x tiles_n workgroups in the dense kernels' tile order, each fetching the
+ *     128 rows of its row tile from x (tiles_m * 128 rows of K bytes, x_bytes in all) and / or its 64 weight rows from w
+ *     (tiles_n * 64 rows, w_bytes), 128 bytes of K per step, five steps ahead.  which: 1 activations only, 2 weights
+ *     only, 3 both.  K a multiple of 128.  The duration is what the memory system allows the tile kernel on operands of
+ *     that shape.
  */
 int mslk_amd_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, void* stream);
 int mslk_amd_debug_mfma_loop(const void* operands, int form, int iters, int workgroups, void* sink, void* stream);
+int mslk_amd_debug_tile_streams(const void* x, int64_t x_bytes, const void* w, int64_t w_bytes, int64_t K, int tiles_m, int tiles_n,
+                                int which, void* stream);
 
 /*
  * Where the time of one dense launch goes: the 256 x 256 tile kernel of mslk_amd_f8f8bf16_rowwise (one tile per

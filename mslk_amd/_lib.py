@@ -59,6 +59,7 @@ SIGNATURES = {
     "mslk_amd_debug_dispatch_name": (c_char_p, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_int]),
     "mslk_amd_debug_stream_read": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
     "mslk_amd_debug_mfma_loop": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "mslk_amd_debug_tile_streams": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
     "mslk_amd_debug_gemm_phases": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p]),
 }
 

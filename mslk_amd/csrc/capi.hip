@@ -452,6 +452,18 @@ int mslk_amd_debug_mfma_loop(const void* operands, int form, int iters, int work
   return check_hip(launch_debug_mfma_loop(operands, form, iters, workgroups, sink, (hipStream_t)stream), "mfma loop launch");
 }
 
+int mslk_amd_debug_tile_streams(const void* x, int64_t x_bytes, const void* w, int64_t w_bytes, int64_t K, int tiles_m, int tiles_n,
+                                int which, void* stream) {
+  if (which < 1 || which > 3) return fail("debug_tile_streams: which must be 1 (activations), 2 (weights) or 3 (both)");
+  if (K < 128 || K % 128 != 0 || K > (1 << 20)) return fail("debug_tile_streams: K must be a multiple of 128 in 128 .. 2^20, got %lld", (long long)K);
+  if (tiles_m <= 0 || tiles_n <= 0 || (int64_t)tiles_m * tiles_n > (1 << 20)) return fail("debug_tile_streams: tiles_m * tiles_n must be in 1 .. 2^20");
+  if (x_bytes < (int64_t)tiles_m * 128 * K || w_bytes < (int64_t)tiles_n * 64 * K)
+    return fail("debug_tile_streams: x must hold tiles_m * 128 rows of K bytes and w tiles_n * 64 rows");
+  if (!x || !w || reinterpret_cast<uintptr_t>(x) % 16 != 0 || reinterpret_cast<uintptr_t>(w) % 16 != 0)
+    return fail("debug_tile_streams: x and w must be 16-byte aligned device pointers");
+  return check_hip(launch_debug_tile_streams(x, w, (int)K, tiles_m, tiles_n, which, (hipStream_t)stream), "tile streams launch");
+}
+
 int mslk_amd_debug_gemm_phases(const void* xq, const void* wq, const float* x_scale, const float* w_scale, void* y, int64_t M,
                                int64_t N, int64_t K, uint64_t* stamps, void* stream) {
   if (M <= 0 || N <= 0 || M % 256 != 0 || N % 256 != 0 || M > (1 << 20) || N > (1 << 20))

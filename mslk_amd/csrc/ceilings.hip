@@ -50,6 +50,57 @@ __global__ __launch_bounds__(256) void stream_dma_kernel(const uint8_t* __restri
   (void)sink;
 }
 
+// The two operand streams of the 128 x 64 tile kernel's K loop without its LDS reads and multiplies: a workgroup fetches
+// the 128 activation rows of its row tile (shared with every workgroup of that row tile: L2 hits) and its own 64 weight
+// rows (read by the row tiles of one panel only: HBM), 128 bytes of K per step through a ring of six 24 KiB stages, five
+// steps ahead, a wave-level wait and a workgroup barrier per step -- the access pattern, tile order and pipeline depth
+// of dense_tiled<128, 64, ring 6>.  WHICH: 1 activations only, 2 weights only, 3 both.  What the launch takes is what
+// the memory system allows that kernel on the same operands.
+template <int WHICH>
+__global__ __launch_bounds__(256) void tile_streams_kernel(const uint8_t* __restrict__ x, const uint8_t* __restrict__ w, int K,
+                                                           int tiles_m, int tiles_n) {
+  constexpr int NS = 6, STAGE = 24 * 1024, XL = 4, WL = 2;    // per wave and step: four activation loads, two weight loads
+  constexpr int PER = ((WHICH & 1) ? XL : 0) + ((WHICH & 2) ? WL : 0);
+  __shared__ __attribute__((aligned(1024))) char lds[NS * STAGE];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // tile order of the dense kernels: XCD x (workgroup id mod 8) takes a contiguous slice of the list of panels of up to
+  // four row tiles, column-major inside a panel
+  const int ntiles = tiles_m * tiles_n, per_xcd = (ntiles + 7) / 8;
+  const int t = (blockIdx.x % 8) * per_xcd + blockIdx.x / 8;
+  if (t >= ntiles || (int)(blockIdx.x / 8) >= per_xcd) return;
+  const int panel = 4 * tiles_n, first_m = (t / panel) * 4;
+  const int rows = tiles_m - first_m < 4 ? tiles_m - first_m : 4;
+  const int tm = first_m + (t % panel) % rows, tn = (t % panel) / rows;
+  const uint8_t* xb = x + (int64_t)tm * 128 * K + (lane >> 3) * (int64_t)K + (lane & 7) * 16;   // a load covers 8 rows x 128 bytes
+  const uint8_t* wb = w + (int64_t)tn * 64 * K + (lane >> 3) * (int64_t)K + (lane & 7) * 16;
+  const int KT = K / 128;
+  auto issue = [&](int kt) {
+    char* st = lds + (kt % NS) * STAGE + wave * (STAGE / 4);
+    if constexpr ((WHICH & 1) != 0) {
+#pragma unroll
+      for (int q = 0; q < XL; ++q)
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(xb + (int64_t)(wave * XL + q) * 8 * K + kt * 128), (lds_ptr_t)(st + q * 1024), 16, 0, 0);
+    }
+    if constexpr ((WHICH & 2) != 0) {
+#pragma unroll
+      for (int q = 0; q < WL; ++q)
+        __builtin_amdgcn_global_load_lds((gbl_ptr_t)(wb + (int64_t)(wave * WL + q) * 8 * K + kt * 128), (lds_ptr_t)(st + (XL + q) * 1024), 16, 0, 0);
+    }
+  };
+  for (int i = 0; i < NS - 1 && i < KT; ++i) issue(i);
+  for (int kt = 0; kt < KT; ++kt) {
+    if (kt + NS - 1 < KT) {
+      issue(kt + NS - 1);
+      constexpr int PENDING = (NS - 1) * PER;   // the loads of the five steps ahead may still be in flight
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (PENDING & 15) | ((PENDING >> 4) << 14));
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0)
+    }
+    __builtin_amdgcn_s_barrier();
+  }
+}
+
 // Register-only MFMA loops on the operands at `src` (4096 fragments of 32 bytes per lane slot): 64 (16x16x128) or 32
 // (32x32x64) independent accumulators per wave, the wave tile of the GEMM (128 x 128 x 128 per iteration), one wave per
 // SIMD.  No memory traffic inside the loop: what it sustains is the matrix cores' rate at the clock the power limit grants
@@ -118,6 +169,16 @@ hipError_t launch_debug_stream_read(const void* src, int64_t bytes, int mode, in
   if (mode == 0) stream_read_kernel<<<workgroups, 256, 0, s>>>(static_cast<const v4i*>(src), bytes / 16, static_cast<int*>(sink));
   else if (mode == 1) stream_dma_kernel<false><<<workgroups, 256, 0, s>>>(static_cast<const uint8_t*>(src), bytes / 1024, static_cast<int*>(sink));
   else stream_dma_kernel<true><<<workgroups, 256, 0, s>>>(static_cast<const uint8_t*>(src), bytes / 1024, static_cast<int*>(sink));
+  return hipGetLastError();
+}
+
+hipError_t launch_debug_tile_streams(const void* x, const void* w, int K, int tiles_m, int tiles_n, int which, hipStream_t s) {
+  const int grid = (tiles_m * tiles_n + 7) / 8 * 8;
+  const uint8_t* xp = static_cast<const uint8_t*>(x);
+  const uint8_t* wp = static_cast<const uint8_t*>(w);
+  if (which == 1) tile_streams_kernel<1><<<grid, 256, 0, s>>>(xp, wp, K, tiles_m, tiles_n);
+  else if (which == 2) tile_streams_kernel<2><<<grid, 256, 0, s>>>(xp, wp, K, tiles_m, tiles_n);
+  else tile_streams_kernel<3><<<grid, 256, 0, s>>>(xp, wp, K, tiles_m, tiles_n);
   return hipGetLastError();
 }
 

@@ -22,6 +22,9 @@ hipError_t launch_cast_e4m3fn(const float* in, int64_t n, void* out, hipStream_t
 // at `operands`.
 hipError_t launch_debug_stream_read(const void* src, int64_t bytes, int mode, int workgroups, void* sink, hipStream_t s);
 hipError_t launch_debug_mfma_loop(const void* operands, int form, int iters, int workgroups, void* sink, hipStream_t s);
+// The operand streams of a 128 x 64 tile K loop alone (which: 1 activations, 2 weights, 3 both); x holds tiles_m * 128 rows
+// of K bytes, w tiles_n * 64 rows; K a multiple of 128.
+hipError_t launch_debug_tile_streams(const void* x, const void* w, int K, int tiles_m, int tiles_n, int which, hipStream_t s);
 
 // Fused producers of quantized activations (fused_quant.hip).
 enum FusedQuantOp : int { kFusedSiluMul = 0, kFusedGatherScale = 1 };

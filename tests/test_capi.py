@@ -47,6 +47,12 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert L.mslk_amd_f8f8bf16_rowwise_batched(None, None, None, None, None, 1, 2, 4, 8, 16, None, None) != 0
     assert b"bias" in L.mslk_amd_last_error()
     assert L.mslk_amd_f8f8bf16_rowwise_batched(None, None, None, None, None, 0, 0, 4, 8, 16, None, None) == 0
+    assert L.mslk_amd_debug_tile_streams(None, 0, None, 0, 8192, 2, 128, 4, None) != 0
+    assert b"which" in L.mslk_amd_last_error()
+    assert L.mslk_amd_debug_tile_streams(None, 0, None, 0, 100, 2, 128, 3, None) != 0
+    assert b"multiple of 128" in L.mslk_amd_last_error()
+    assert L.mslk_amd_debug_tile_streams(None, 2 * 128 * 256 - 1, None, 128 * 64 * 256, 256, 2, 128, 3, None) != 0
+    assert b"must hold" in L.mslk_amd_last_error()
     # empty problems are a successful no-op and touch no pointer
     assert L.mslk_amd_f8f8bf16_rowwise(None, None, None, None, None, 0, None, 0, 4, 4, None, 0, None) == 0
     assert L.mslk_amd_quantize_fp8_row(None, 0, 0, 16, 16, None, 16, None, None, None) == 0

@@ -133,6 +133,24 @@ def test_measuring_build_of_the_tile_kernel_gives_the_product_bits_and_ordered_s
     assert b"multiples of 256" in L.mslk_amd_last_error()
 
 
+@pytest.mark.parametrize("tiles_m,tiles_n,K", [(2, 128, 1024), (1, 3, 128), (5, 7, 640)])
+def test_operand_stream_probe_reads_its_operands_and_writes_nothing(tiles_m, tiles_n, K):
+    """mslk_amd_debug_tile_streams issues the loads of the 128 x 64 tile kernel's K loop and nothing else: every variant
+    runs to completion on operands of exactly the stated size (tile counts that do and do not fill the grid's multiple of
+    8, K loops shorter and longer than the ring), and the operands and a guard region behind them are unchanged."""
+    from mslk_amd import _lib
+    g = torch.Generator().manual_seed(tiles_m * 100 + tiles_n)
+    nx, nw = tiles_m * 128 * K, tiles_n * 64 * K
+    buf = torch.randint(0, 255, (nx + nw + 4096,), dtype=torch.uint8, generator=g).to(DEV)
+    before = buf.clone()
+    L = _lib.lib()
+    for which in (1, 2, 3):
+        _lib.check(L.mslk_amd_debug_tile_streams(buf.data_ptr(), nx, buf.data_ptr() + nx, nw, K, tiles_m, tiles_n, which,
+                                                 torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert torch.equal(buf, before)
+
+
 def test_identity_and_one_hot_weights_select_dequantized_activations():
     g = torch.Generator().manual_seed(9)
     M, K = 300, 512
