@@ -82,6 +82,8 @@ int device_compute_units();
 // Shape classes; each returns hipErrorInvalidValue when the shape is outside what it supports.
 bool dense_tiled_supports(const GemmProblem& p);
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s);
+// Its branch for pre-shuffled weights (a translation unit of its own); cus: device_compute_units().
+hipError_t launch_dense_tiled_preshuffled(const GemmProblem& p, int cus, hipStream_t s);
 bool skinny_supports(const GemmProblem& p);
 // Row-major weights at least this wide take the short LDS tiles instead of the weight-streaming kernel for 8 < M <= 64
 // (measured crossover: streaming wins at N = 4096, tiles from N = 5120 on).
