@@ -339,9 +339,13 @@ hipError_t launch_device_layout(const DeviceGroups& p, hipStream_t s) {
 // row tiles shares it (59 us), and a ragged tile with a quarter of the rows takes about three quarters of a full one.
 // The groups are therefore cut into panels of up to kGroupM row tiles (all column tiles of those rows: the unit inside
 // which operand tiles are shared through the L2), every panel gets a cost from that model, the panels are dealt to the
-// XCDs longest first onto the least loaded one, and inside an XCD the panels with the cheapest tiles come last, so
-// that the last pass over the CUs is a short one.  A panel is just another group descriptor (same weights, row range
-// of the activations and of the output); when the panels would not fit the descriptor table, whole groups are dealt.
+// XCDs longest first onto the least loaded one -- every XCD gets dear and cheap panels alike; all the weight-bound ones
+// on two XCDs was measured and is 7 - 13 % slower --, and inside an XCD the panels with the cheapest tiles come last, so
+// that the last pass over the CUs is a short one.  Where the deal leaves an XCD more than 3 % of an even share away from
+// it (few panels: one or two big groups), the boundary between two XCDs moves into a panel instead: its tiles are
+// ordered column by column, so the two XCDs get column ranges of it.  A panel is just another group descriptor (same
+// weights, row range of the activations and of the output); when the panels would not fit the descriptor table, whole
+// groups are dealt.
 hipError_t launch_grouped_tiled(const GroupTable& in, hipStream_t s) {
   if (in.total_tiles <= 0 || in.count <= 0) return hipSuccess;
   constexpr int BM = 256, BN = 256;
@@ -378,12 +382,14 @@ hipError_t launch_grouped_tiled(const GroupTable& in, hipStream_t s) {
   std::stable_sort(order, order + n, [&](int a, int b) { return chunks[a].cost > chunks[b].cost; });
   int bin_of[kMaxGroupsPerLaunch];
   float load[kXcds] = {};
+  double total = 0.0;
   for (int i = 0; i < n; ++i) {
     int best = 0;
     for (int x = 1; x < kXcds; ++x)
       if (load[x] < load[best]) best = x;
     bin_of[order[i]] = best;
     load[best] += chunks[order[i]].cost;
+    total += chunks[order[i]].cost;
   }
   // inside an XCD: panels whose cheapest tile is expensive first
   std::stable_sort(order, order + n, [&](int a, int b) {
@@ -392,11 +398,9 @@ hipError_t launch_grouped_tiled(const GroupTable& in, hipStream_t s) {
   });
   GroupTable t;
   t.count = n;
-  int tiles = 0, longest = 0, x = 0;
-  t.xcd_begin[0] = 0;
+  int tiles = 0;
   for (int i = 0; i < n; ++i) {
     const Chunk& c = chunks[order[i]];
-    while (x < bin_of[order[i]]) t.xcd_begin[++x] = tiles;
     const GroupDesc& d = in.g[c.group];
     GroupDesc& o = t.g[i];
     o = d;
@@ -407,8 +411,54 @@ hipError_t launch_grouped_tiled(const GroupTable& in, hipStream_t s) {
     o.tile_begin = tiles;
     tiles += c.tiles;
   }
-  while (x < kXcds) t.xcd_begin[++x] = tiles;
   t.total_tiles = tiles;
+  // XCD x works on tiles [xcd_begin[x], xcd_begin[x + 1]).  Two plans: the deal (whole panels per XCD), and the same list
+  // cut into eight runs of equal cost, a cut falling wherever the running cost reaches the next eighth.  Each is priced as
+  // the slowest XCD's passes over its CUs (tiles / CUs of an XCD, rounded up) times the mean cost of its tiles; the deal
+  // keeps every XCD at whole panels -- multiples of the column count, which full passes are made of -- and wins whenever
+  // there are panels enough (measured: cutting cfg4 evenly by cost costs 7 %, because the cuts leave partial passes);
+  // the even cut wins when the deal leaves XCDs idle (one group of 1024 rows: 189 -> 47 us).
+  const int cus_per_xcd = device_compute_units() / kXcds;
+  int plan_a[kXcds + 1], plan_b[kXcds + 1];
+  plan_a[0] = plan_b[0] = 0;
+  plan_a[kXcds] = plan_b[kXcds] = tiles;
+  const double share = total / kXcds;
+  for (int x = 0, i = 0; x + 1 < kXcds; ++x) {
+    while (i < n && bin_of[order[i]] <= x) ++i;
+    plan_a[x + 1] = i < n ? t.g[i].tile_begin : tiles;
+    const double target = share * (x + 1);
+    double done = 0.0;
+    int j = 0;
+    while (j + 1 < n && done + chunks[order[j]].cost < target) done += chunks[order[j++]].cost;
+    const Chunk& c = chunks[order[j]];
+    int in_chunk = (int)((target - done) / ((double)c.cost / c.tiles) + 0.5);   // a chunk's tiles are taken to cost the same
+    in_chunk = in_chunk < 0 ? 0 : (in_chunk > c.tiles ? c.tiles : in_chunk);
+    const int at = t.g[j].tile_begin + in_chunk;
+    plan_b[x + 1] = at < plan_b[x] ? plan_b[x] : at;
+  }
+  auto price = [&](const int* begin) {
+    double worst = 0.0;
+    int j = 0;
+    for (int x = 0; x < kXcds; ++x) {
+      const int lo = begin[x], hi = begin[x + 1];
+      if (hi <= lo) continue;
+      double cost = 0.0;
+      while (j < n && t.g[j].tile_begin + chunks[order[j]].tiles <= lo) ++j;
+      for (int k = j; k < n && t.g[k].tile_begin < hi; ++k) {
+        const Chunk& c = chunks[order[k]];
+        const int from = t.g[k].tile_begin > lo ? t.g[k].tile_begin : lo;
+        const int to = t.g[k].tile_begin + c.tiles < hi ? t.g[k].tile_begin + c.tiles : hi;
+        cost += (double)c.cost / c.tiles * (to - from);
+      }
+      const int passes = (hi - lo + cus_per_xcd - 1) / cus_per_xcd;
+      const double time = cost / (hi - lo) * passes;
+      if (time > worst) worst = time;
+    }
+    return worst;
+  };
+  const bool even_cut = price(plan_b) < 0.9 * price(plan_a);
+  for (int x = 0; x <= kXcds; ++x) t.xcd_begin[x] = even_cut ? plan_b[x] : plan_a[x];
+  int longest = 0;
   for (int i = 0; i < kXcds; ++i)
     if (t.xcd_begin[i + 1] - t.xcd_begin[i] > longest) longest = t.xcd_begin[i + 1] - t.xcd_begin[i];
   grouped_tiled_kernel<256, 256><<<longest * kXcds, 256, 0, s>>>(t);

@@ -77,10 +77,12 @@ def _groups(ms, N, K, g):
     return xi, wi, xs, ws
 
 
-@pytest.mark.parametrize("ms,N,K", [(ROWSKIP_256, 768, 640), (ROWSKIP_256[:9], 1024, 528), ([3] * 70, 512, 512)])
+@pytest.mark.parametrize("ms,N,K", [(ROWSKIP_256, 768, 640), (ROWSKIP_256[:9], 1024, 528), ([3] * 70, 512, 512),
+                                    ([1100], 2304, 512), ([2100, 300], 1024, 640), ([257, 0, 1025], 4096, 512)])
 def test_tensorlist_grouped_exact(ms, N, K):
     """grouped_tiled_kernel: 256 x 256 tiles, reduced K loops (1/4, 1/2, 3/4 of the m fragments) with the fragments dealt
-    to the wave rows round-robin, panels of four row tiles, a K tail in the second case, more than 64 groups in the third."""
+    to the wave rows round-robin, panels of four row tiles, a K tail in the second case, more than 64 groups in the third;
+    one to three groups in the others: fewer panels than XCDs, so the launcher cuts panels between XCDs."""
     g = torch.Generator().manual_seed(sum(ms) + N + K)
     xi, wi, xs, ws = _groups(ms, N, K, g)
     dev = lambda ts, f8=False: [(t.to(F8) if f8 else t).to(DEV) for t in ts]
