@@ -212,6 +212,14 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // half full -- fewer LDS bytes per MFMA than 128 x 128 tiles and half the row granularity of 256 x 256
   // (N = K = 8192, M = 1024: 66.4 -> 59.7 us; N = K = 4096, M = 2048: 31.6 -> 29.0 us; N = 57344, K = 8192, M = 128:
   // 118.5 -> 108.6 us).
+  // 192 x 128 tiles (wave tile 96 x 64, three ring buffers) when the 128 x 128 tiles no longer fit one per CU and these
+  // do: with at most one tile per CU the launch takes what one tile takes, and a tile's K step costs what it moves
+  // into the LDS -- 40 KiB here against 48 KiB for 128 x 256 (M = 768, N = 7168, K = 6144: 45.8 -> 36.7 us;
+  // M = 768, N = 6144, K = 7168: 47.5 -> 40.6; M = 768, N = K = 8192: 54.6 -> 49.0).
+  if (small_tiles > cus && big_tiles <= cus / 2) {
+    const int64_t tiles19 = (int64_t)((p.M + 191) / 192) * ((p.N + 127) / 128);
+    if (tiles19 <= cus) return launch_tiled_shape<TileShape<192, 128, 2, 2, 3>, false>(p, s);
+  }
   {
     const int64_t rows128 = (p.M + 127) / 128;
     const int64_t tiles12 = rows128 * ((p.N + 255) / 256);
@@ -221,7 +229,14 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // Otherwise 256 x 256 tiles from 129 tiles on: the 128 x 256 tiles would then need two passes and the co-resident
   // 128 x 128 tiles more than two per CU (N = 6144, M = 1536: 144 tiles, K = 8192: 100.0 -> 87.1 us, K = 4096:
   // 48.9 -> 39.5 us).
-  if (big_tiles > cus / 2) return launch_tiled_shape<TileShape<256, 256>, false, 1>(p, s);
+  if (big_tiles > cus / 2) {
+    // 192 x 256 tiles (wave tile 96 x 128, two-plus-three buffers) where they still fit one per CU: a quarter less work
+    // per tile on a third more CUs (M = 1536, N = K = 8192: 80.0 -> 76.3 us; M = 768, N = 16384, K = 8192: 85.0 -> 76.3;
+    // M = 1344, N = 8192, K = 4096: 41.5 -> 37.5)
+    const int64_t tiles19 = (int64_t)((p.M + 191) / 192) * ((p.N + 255) / 256);
+    if (tiles19 <= cus && p.K >= 2048) return launch_tiled_shape<TileShape<192, 256>, false>(p, s);
+    return launch_tiled_shape<TileShape<256, 256>, false, 1>(p, s);
+  }
   // M > 64 with at most one 64 x 64 tile per CU: such tiles (four waves stacked along M, five ring buffers, two
   // workgroups per CU) wherever they cover at least as many CUs as the 128-row tiles below would, in a single pass:
   // rows 65 ... 128 then do not cost a second, half-empty 128-row tile's worth of activation traffic (N = K = 8192,

@@ -172,7 +172,10 @@ DISPATCH_TABLE = [
     ((8192, 8192, 8192, 0, 0, 0, 1), "dense_persistent<256,256> tiles=1024 workgroups=256"),
     ((2304, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256 + dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
     ((2048, 4096, 4096, 0, 0, 0, 1), "dense_tiled<128,256,waves=2x2,ring=3> tiles=256"),
-    ((1536, 6144, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=144"),
+    ((1536, 6144, 8192, 0, 0, 0, 1), "dense_tiled<192,256,waves=2x2,ring=0> tiles=192"),                     # 144 tiles of 256 x 256: 192-row tiles still fit one per CU
+    ((1728, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=224"),                     # ... and here they do not
+    ((1536, 6144, 1024, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=144"),                     # short K keeps the fused epilogue of the 256 x 256 tiles
+    ((768, 7168, 6144, 0, 0, 0, 1), "dense_tiled<192,128,waves=2x2,ring=3> tiles=224"),                      # 128 x 128 tiles would need two passes
     ((512, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,128,waves=2x2,ring=5> tiles=256"),
     ((256, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
     ((128, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=256"),
