@@ -201,9 +201,13 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // at N = 5120 ... 57344.  Above N = 8192 the 64 x 32 tiles of 32 < M <= 64 no longer fit one per CU and the CUs that
   // hold two move twice the activation bytes; 64 x 64 tiles halve the tile count and the activation traffic
   // (N = 10240, K = 8192, M = 64: 33.3 -> 28.3 us; N = 57344, K = 4096, M = 64: 68.4 -> 55.5 us).
+  // The same holds for fewer rows on wider weights (M = 32: N = 10240, K = 8192 21.4 -> 20.0 us, N = 32768, K = 7168
+  // 46.4 -> 39.0 us; M = 12, N = 28672, K = 8192 45.3 -> 39.8 us), down to M <= 16, where the 32 x 32 tiles hold up to
+  // N = 16384 (N = 14336, K = 8192: 22.8 against 23.4 us).
   if (p.M <= 64 && p.N >= kShortTileMinN) {
-    if (p.M <= 32 && p.N <= 16384) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false, 2>(p, s);
-    if (p.M <= 32 || p.N <= 8192) return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false, 2>(p, s);
+    if (p.M <= 32 && p.N <= (p.M <= 16 ? 16384 : 8192)) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false, 2>(p, s);
+    if (p.M > 32 ? p.N <= 8192 : (p.N > 16384 && p.N < 24576))   // M = 9, N = 22016, K = 8192: 36.8 against 38.9 us on 64 x 64 tiles
+      return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false, 2>(p, s);
     return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false, 1>(p, s);
   }
   if (big_tiles > cus) return launch_persistent_shape<TileShape<256, 256>, false>(p, cus, s);

@@ -168,6 +168,9 @@ DISPATCH_TABLE = [
     ((64, 4096, 14336, 0, 0, 0, 1), "skinny_lds<m_frags=4,n_frags=1,steps=1> workgroups=256"),
     ((8, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),                  # last M of the streaming kernel on wide weights
     ((9, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> weights streamed tiles=256"),
+    ((32, 10240, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> weights streamed tiles=160"),        # M <= 32 on wider weights
+    ((9, 22016, 8192, 0, 0, 0, 1), "dense_tiled<64,32,waves=4x1,ring=6> weights streamed tiles=688"),
+    ((32, 32768, 7168, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> weights streamed tiles=512"),
     ((3, 1000, 272, 0, 0, 0, 1), "skinny_registers<m_frags=1,n_frags=1,steps=8> workgroups=63"),              # K % 1024 != 0
     ((8192, 8192, 8192, 0, 0, 0, 1), "dense_persistent<256,256> tiles=1024 workgroups=256"),
     ((2304, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256 + dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),

@@ -266,7 +266,7 @@ def test_preshuffled_tiles_exact(M, N, K, fp16_out):
 
 
 @pytest.mark.parametrize("M,N,K", [(1024, 8192, 384), (2048, 4096, 272), (96, 8192, 512), (128, 4096, 400), (40, 8192, 1040),
-                                   (24, 12288, 256), (64, 16384, 384), (1536, 6144, 144),
+                                   (24, 12288, 256), (16, 12288, 256), (24, 20480, 384), (64, 16384, 384), (1536, 6144, 144),
                                    (1000, 5000, 528), (768, 7168, 256), (960, 6144, 128),       # 192 x 128 tiles, ring of three
                                    (1536, 6144, 2064), (1500, 6100, 2048)])                      # 192 x 256 tiles, two-plus-three buffers
 def test_ring_and_short_tiles_exact(M, N, K):
