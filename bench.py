@@ -173,9 +173,18 @@ class CApi:
         M = xq.shape[0]
         N, K = wq.shape
         bcode = 0 if bias is None else (1 if bias.dtype.itemsize == 4 else 2)
+        # the workspace the library asks for (K-split shapes), allocated once per size and outside every timed region,
+        # as the caching allocator does for the operator
+        need = self.L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+        wsp = None
+        if need:
+            import torch
+            if getattr(self, "_wsp", None) is None or self._wsp.numel() < need:
+                self._wsp = torch.empty(need, dtype=torch.uint8, device=xq.device)
+            wsp = self._wsp.data_ptr()
         self.check(self.L.mslk_amd_f8f8bf16_rowwise(xq.data_ptr(), wq.data_ptr(), xs.data_ptr(), ws.data_ptr(),
                                                     None if bias is None else bias.data_ptr(), bcode, y.data_ptr(),
-                                                    M, N, K, None, 0, self.stream))
+                                                    M, N, K, wsp, need, self.stream))
 
     def grouped_call(self, xq, wq, xs, ws, ys):
         """Pre-marshalled TensorList call: returns a closure that only crosses the C ABI."""

@@ -131,13 +131,19 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
  * csrc/gemm/cutlass/f8f8bf16_rowwise/f8f8bf16_rowwise_common.cuh:150-198).
  * M, N or K equal to 0 writes zeros to Y (fp8fp8bf16_rowwise_gemm.hip:531-534).
  * `workspace` (device memory, 16-byte aligned) is optional and only used when
- * mslk_amd_f8f8bf16_rowwise_workspace_bytes(M,N,K) > 0, i.e. when K is not a multiple of 16: the call then copies both
- * operands into workspace rows of K rounded up to 16 (zero tail) and runs the MFMA kernels on the copies (the CK
- * instances of the reference pad K inside the kernel, fp8_rowwise_common.h:109-110 `GemmSpecialization::MNKPadding`).
- * An operand base pointer that is not 16-byte aligned is handled the same way if the workspace holds
- * (M + N) * round_up(K, 16) bytes.  Without a workspace (null or too small) such operands still give the same results
- * through a scalar kernel that is orders of magnitude slower.  The workspace needs no initialisation and holds nothing between calls; calls that
- * share one workspace must not overlap.
+ * mslk_amd_f8f8bf16_rowwise_workspace_bytes(M,N,K) > 0.  Two cases:
+ *   - K is not a multiple of 16: the call copies both operands into workspace rows of K rounded up to 16 (zero tail) and
+ *     runs the MFMA kernels on the copies (the CK instances of the reference pad K inside the kernel,
+ *     fp8_rowwise_common.h:109-110 `GemmSpecialization::MNKPadding`).  An operand base pointer that is not 16-byte aligned
+ *     is handled the same way if the workspace holds (M + N) * round_up(K, 16) bytes.  Without a workspace (null or too
+ *     small) such operands still give the same results through a scalar kernel that is orders of magnitude slower.
+ *   - few output tiles and a long K (64 < M, at most 128 tiles of 64 x 64 on a whole MI355X, K >= 6144 ... 8192; the
+ *     reference's instances for such shapes split K as well, fp8_rowwise_common.h:168-204 `KBatch`): the call cuts K into
+ *     2 ... 8 slices, whose fp32 sums go into the workspace (slices * M * N floats), and a second launch adds them and
+ *     applies scales, bias and the conversion -- two to three times faster where the unsplit kernels would leave most
+ *     CUs idle.  Without a workspace the unsplit kernels run; on operands whose products and sums are exact in fp32
+ *     both give the same bits, otherwise they differ by the rounding of a different summation order.
+ * The workspace needs no initialisation and holds nothing between calls; calls that share one workspace must not overlap.
  */
 int mslk_amd_f8f8bf16_rowwise(const void* xq, const void* wq, const float* x_scale, const float* w_scale,
                               const void* bias, int bias_dtype, void* y,
@@ -153,7 +159,8 @@ size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K
  * holds it until the process ends); the call allocates and frees nothing.  Shapes whose copies do not fit,
  * (M + N) * round_up(K, 16) > MSLK_AMD_STATIC_SCRATCH_BYTES, are rejected with an error.  The array needs no
  * initialisation (the copies overwrite every byte they later read), but all calls on one GPU share it: calls that
- * overlap on one GPU (different streams, or threads) race.  Shapes that need no copies never touch the array.
+ * overlap on one GPU (different streams, or threads) race.  Shapes that the library splits along K (see above) put the
+ * sums of their slices into the same array when they fit, and run unsplit when they do not.  Other shapes never touch it.
  * The first call on a device that needs the copies looks the array's address up (hipGetSymbolAddress; not a stream
  * operation) and is also the moment HIP commits the array's device memory; a caller that captures graphs or measures
  * memory makes that first call outside the capture / before the measurement.

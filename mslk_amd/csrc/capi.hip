@@ -174,9 +174,13 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
 // K that is not a multiple of 16: the operand rows cannot be fetched by the 16-byte loads of the MFMA kernels.  With a
 // workspace the call copies both operands into rows of K rounded up to 16 (zero tail: code 0x00 is +0) and runs the
 // ordinary kernels on the copies; without one it falls back to the scalar kernel, which is orders of magnitude slower.
+// K a multiple of 16 on a shape with few output tiles and a long K: with a workspace of slices * M * N floats the call
+// splits K (gemm_splitk.hip); without one it runs the ordinary kernels.
 size_t mslk_amd_f8f8bf16_rowwise_workspace_bytes(int64_t M, int64_t N, int64_t K) {
-  if (M <= 0 || N <= 0 || K <= 0 || K % 16 == 0) return 0;
-  return (size_t)((M + N) * ((K + 15) / 16 * 16));
+  if (M <= 0 || N <= 0 || K <= 0 || M > kIntMax || N > kIntMax || K > kIntMax) return 0;
+  if (K % 16 != 0) return (size_t)((M + N) * ((K + 15) / 16 * 16));
+  const SplitKPlan plan = splitk_plan(M, N, K, device_compute_units());
+  return plan.slices > 1 ? (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 
 static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void* xq, const void* wq, const float* x_scale,
@@ -211,10 +215,16 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
       p.K = (int)Kp;
     }
   }
+  const bool tiled_ok = dense_tiled_supports(p);
+  // Few output tiles and a long K: split K when the caller's workspace holds the fp32 sums of every slice.
+  if (!unfetchable && !preshuffled && tiled_ok && workspace && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+    const SplitKPlan plan = splitk_plan(M, N, K, device_compute_units());
+    if (plan.slices > 1 && workspace_bytes >= (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float))
+      return check_hip(launch_splitk(p, plan, static_cast<float*>(workspace), s), "split-K launch");
+  }
   // M <= 64: the weight-streaming kernel, except on wide row-major weights, where short tiles that share their
   // activation rows through LDS win from M = 9 on.  Pre-shuffled weights
   // keep the streaming kernel, whose register-direct weight loads stay ahead up to M = 64.
-  const bool tiled_ok = dense_tiled_supports(p);
   const bool wide = !p.w_preshuffled && p.M > 8 && p.N >= kShortTileMinN;
   if (skinny_supports(p) && !(tiled_ok && wide)) return check_hip(launch_skinny(p, s), "skinny launch");
   if (tiled_ok) return check_hip(launch_dense_tiled(p, s), "tiled launch");
@@ -244,6 +254,14 @@ int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, con
                   "use mslk_amd_f8f8bf16_rowwise with a workspace", op, need, kScratchBytes);
     if (int rc = scratch_of_current_device(&ptr)) return rc;
     bytes = kScratchBytes;
+  } else {
+    // a shape the library would split along K: the fp32 sums of the slices go into the array when they fit (otherwise
+    // the unsplit kernels run, as without a workspace)
+    const size_t need = mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K);
+    if (need > 0 && need <= kScratchBytes) {
+      if (int rc = scratch_of_current_device(&ptr)) return rc;
+      bytes = kScratchBytes;
+    }
   }
   return rowwise_impl(op, 0, 0, xq, wq, x_scale, w_scale, bias, bias_dtype, y, M, N, K, ptr, bytes, stream);
 }

@@ -486,6 +486,37 @@ struct GemmTile {
     epilogue(lds, acc, xs, ws, bias, y, m_rem, n_rem, N);
   }
 
+  // K loop over K bytes of the operand rows, then the raw fp32 sums of the tile to `part` (row pitch ldp floats, already
+  // offset to the tile's first row and column): one slice of a K-split product, scaled and converted by a later pass.
+  // A lane holds 4 consecutive columns of one row per fragment, so full tiles with 16-byte aligned rows store 16 bytes.
+  MSLK_AMD_DEVINL void run_partial(char* lds, const uint8_t* xq_tile, const uint8_t* wq_tile, float* part, int m_rem,
+                                   int n_rem, int ldp, int K, uint32_t ld) {
+    static_assert(TS::FM * TS::FN * 4 < 256, "tiles whose sums live in vector registers");
+    v4f acc[TS::FN][TS::FM];
+    accumulate_rows(lds, xq_tile, wq_tile, m_rem, n_rem, K, ld, acc);
+    const int lane = threadIdx.x & 63, wave = wave_id();
+    const int row0 = (wave / TS::WN) * (TS::kBM / TS::WM) + (lane & 15);
+    const int col0 = (wave % TS::WN) * (TS::kBN / TS::WN) + 4 * (lane >> 4);
+    const bool vec = (ldp & 3) == 0 && (reinterpret_cast<uintptr_t>(part) & 15) == 0;
+#pragma unroll
+    for (int tm = 0; tm < TS::FM; ++tm) {
+      const int m = row0 + tm * 16;
+      if (m >= m_rem) continue;
+#pragma unroll
+      for (int tn = 0; tn < TS::FN; ++tn) {
+        const int n = col0 + tn * 16;
+        float* dst = part + (int64_t)m * ldp + n;
+        if (vec && n + 3 < n_rem) {
+          *reinterpret_cast<float4*>(dst) = make_float4(acc[tn][tm][0], acc[tn][tm][1], acc[tn][tm][2], acc[tn][tm][3]);
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (n + r < n_rem) dst[r] = acc[tn][tm][r];
+        }
+      }
+    }
+  }
+
   // Whether run_interior() may take the tile: every row and column valid, 16-byte aligned rows of Y and scale / bias
   // vectors, K a positive multiple of the K step.
   MSLK_AMD_DEVINL static bool interior_ok(const float* ws, const void* bias, const uint16_t* y, int m_rem, int n_rem, int N, int K) {

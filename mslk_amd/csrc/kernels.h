@@ -84,6 +84,14 @@ bool dense_tiled_supports(const GemmProblem& p);
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s);
 // Its branch for pre-shuffled weights (a translation unit of its own); cus: device_compute_units().
 hipError_t launch_dense_tiled_preshuffled(const GemmProblem& p, int cus, hipStream_t s);
+// K-split form for shapes with few output tiles and a long K (gemm_splitk.hip): `slices` workgroups per tile of edge
+// `tile` write fp32 sums to a workspace of slices * M * N floats, a second launch reduces, scales and converts.
+struct SplitKPlan {
+  int tile;     // 64
+  int slices;   // 1: the shape is not split
+};
+SplitKPlan splitk_plan(int64_t M, int64_t N, int64_t K, int cus);
+hipError_t launch_splitk(const GemmProblem& p, const SplitKPlan& plan, float* part, hipStream_t s);
 bool skinny_supports(const GemmProblem& p);
 // Row-major weights at least this wide take the short LDS tiles instead of the weight-streaming kernel for 8 < M <= 64
 // (measured crossover: streaming wins at N = 4096, tiles from N = 5120 on).

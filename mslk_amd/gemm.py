@@ -137,6 +137,12 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, o
         wsp_bytes = (M + N) * ((K + 15) // 16 * 16)
         wsp = torch.empty(wsp_bytes, dtype=torch.uint8, device=XQ.device)
         wsp_ptr = wsp.data_ptr()
+    else:
+        # few output tiles and a long K: the library splits K when it is given room for the fp32 sums of the slices
+        wsp_bytes = _lib.lib().mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+        if wsp_bytes:
+            wsp = torch.empty(wsp_bytes, dtype=torch.uint8, device=XQ.device)
+            wsp_ptr = wsp.data_ptr()
     with _on_device(XQ.device):
         fn = _lib.lib().mslk_amd_f8f8f16_rowwise if out_dtype == torch.float16 else _lib.lib().mslk_amd_f8f8bf16_rowwise
         _lib.check(fn(XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),

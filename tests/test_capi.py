@@ -29,6 +29,8 @@ def test_library_exports_every_declared_symbol():
         assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
     assert L.mslk_amd_version().decode().startswith("mslk_amd")
     assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(4096, 4096, 4096) == 0
+    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(128, 512, 14336) == 8 * 128 * 512 * 4      # eight K slices of fp32 sums
+    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(64, 512, 14336) == 0                      # M <= 64 is never split
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
@@ -178,7 +180,11 @@ DISPATCH_TABLE = [
     ((1536, 6144, 8192, 0, 0, 0, 1), "dense_tiled<192,256,waves=2x2,ring=0> tiles=192"),                     # 144 tiles of 256 x 256: 192-row tiles still fit one per CU
     ((1728, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=224"),                     # ... and here they do not
     ((1536, 6144, 1024, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=144"),                     # short K keeps the fused epilogue of the 256 x 256 tiles
-    ((768, 7168, 6144, 0, 0, 0, 1), "dense_tiled<192,128,waves=2x2,ring=3> tiles=224"),                      # 128 x 128 tiles would need two passes
+    ((768, 7168, 6144, 0, 0, 0, 1), "dense_tiled<192,128,waves=2x2,ring=3> tiles=224"),
+    ((128, 512, 14336, 0, 0, 0, 1), "splitk_partial<64,64,waves=4x1,ring=5> slices=8 + splitk_reduce"),       # few tiles, long K, workspace given
+    ((128, 512, 14336, 0, 0, 0, 0), "dense_tiled<128,32,waves=4x1,ring=8> weights streamed tiles=16"),         # ... and not given
+    ((128, 4096, 14336, 2, 1, 0, 1), "splitk_partial<64,64,waves=4x1,ring=5> slices=2 + splitk_reduce"),
+    ((128, 4096, 4096, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=128"),                          # K too short to split                      # 128 x 128 tiles would need two passes
     ((512, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,128,waves=2x2,ring=5> tiles=256"),
     ((256, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
     ((128, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=256"),

@@ -279,3 +279,37 @@ def test_ring_and_short_tiles_exact(M, N, K):
     y = torch.ops.mslk.f8f8bf16_rowwise(xi.to(F8).to(DEV), wi.to(F8).to(DEV), xs.to(DEV), ws.to(DEV), bias=bias.bfloat16().to(DEV))
     torch.cuda.synchronize()
     _same_bits(y, _want(xi, wi, xs, ws, bias), f"{M}x{N}x{K}")
+
+
+@pytest.mark.parametrize("fp16_out", [False, True])
+@pytest.mark.parametrize("bias_dtype", [None, torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(128, 512, 8192), (96, 2048, 8192), (300, 518, 6160), (65, 4096, 14336), (512, 1024, 8208)])
+def test_k_split_exact(M, N, K, bias_dtype, fp16_out):
+    """Few output tiles and a long K: with the workspace the library asks for, K is cut into slices whose fp32 sums a
+    second launch adds, scales and converts (ragged rows and columns, a column count that rules out 16-byte accesses, a K
+    tail in the last slice).  Same bits as the product of the codes, and as the unsplit kernels give without a workspace."""
+    from mslk_amd import _lib
+    L = _lib.lib()
+    need = L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+    assert need > 0 and need % (M * N * 4) == 0 and 2 <= need // (M * N * 4) <= 8
+    assert L.mslk_amd_debug_dispatch_name(M, N, K, 0, 0, 0, 1).decode().startswith("splitk_partial<64,64")
+    assert "splitk" not in L.mslk_amd_debug_dispatch_name(M, N, K, 0, 0, 0, 0).decode()
+    g = torch.Generator().manual_seed(M + N + K)
+    xi, wi, xs, ws = _ints(M, K, g), _ints(N, K, g), _pow2(M, g), _pow2(N, g)
+    bias = None if bias_dtype is None else torch.randint(-4, 5, (N,), generator=g).float()
+    want = _want(xi, wi, xs, ws, bias, fp16_out)
+    xq, wq, xsd, wsd = xi.to(F8).to(DEV), wi.to(F8).to(DEV), xs.to(DEV), ws.to(DEV)
+    bd = None if bias is None else bias.to(bias_dtype).to(DEV)
+    op = torch.ops.mslk.f8f8f16_rowwise if fp16_out else torch.ops.mslk.f8f8bf16_rowwise
+    y = op(xq, wq, xsd, wsd, bias=bd)          # the operator passes the workspace
+    torch.cuda.synchronize()
+    _same_bits(y, want, f"split {M}x{N}x{K}")
+    # without a workspace: the ordinary kernels, the same bits
+    y2 = torch.full((M, N), SENTINEL, dtype=want.dtype, device=DEV)
+    fn = L.mslk_amd_f8f8f16_rowwise if fp16_out else L.mslk_amd_f8f8bf16_rowwise
+    _lib.check(fn(xq.data_ptr(), wq.data_ptr(), xsd.data_ptr(), wsd.data_ptr(), None if bd is None else bd.data_ptr(),
+                  0 if bd is None else (1 if bias_dtype == torch.float32 else 2), y2.data_ptr(), M, N, K, None, 0,
+                  torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    _same_bits(y2, want, f"unsplit {M}x{N}x{K}")
+
