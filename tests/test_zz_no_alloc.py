@@ -89,6 +89,20 @@ def test_static_scratch_aligned_shapes_do_not_need_the_array():
     assert torch.equal(got.view(torch.int16).cpu(), want.view(torch.int16).cpu())
 
 
+def test_static_scratch_holds_the_sums_of_a_k_split():
+    # a shape the library splits along K (few output tiles, long K): the fp32 sums of the slices go into the array, as
+    # they go into the workspace of the other entry point -- the same kernels, the same bits (on a whole MI355X the sums
+    # of a split never exceed 4 MiB: at most 128 tiles of 64 x 64 in two slices, or fewer tiles in up to eight)
+    M, N, K = 128, 512, 8192
+    L = _lib.lib()
+    assert 0 < L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K) <= L.mslk_amd_static_scratch_bytes()
+    ops = _operands(M, N, K, seed=9)
+    want = _with_workspace(*ops, M, N, K)
+    got = _static(*ops, M, N, K)
+    torch.cuda.synchronize()
+    assert torch.equal(got.view(torch.int16).cpu(), want.view(torch.int16).cpu())
+
+
 def test_static_scratch_rejects_what_does_not_fit():
     L = _lib.lib()
     cap = L.mslk_amd_static_scratch_bytes()
