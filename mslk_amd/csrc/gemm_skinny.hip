@@ -632,7 +632,13 @@ hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
     if (p.M <= 48) return launch_cfg<3, 2, 4, true>(p, s);
     return launch_cfg<4, 2, 4, true>(p, s);
   }
-  if (p.K % (8 * kStep) == 0) {   // both operands through LDS, all global traffic in full lines
+  // Both operands through LDS, all global traffic in full lines: whole K steps, and when they do not divide evenly among
+  // the eight waves (K % 1024 != 0: 11008, 13824 ...) enough of them that the uneven last batch is a small part --
+  // K = 2560 (20 steps, a batch of M <= 16 is 32) is 39 % slower this way, K = 11008 / 13824 10 - 60 % faster
+  // (M = 48, N = 2560, K = 11008: 26.7 -> 10.6 us; M = 2, N = 22016, K = 11008: 52.0 -> 47.4) except for at most eight
+  // rows on at most 4096 weight rows (M = 1, N = 4096, K = 11008: 10.3 against 11.1 us).
+  const bool even = p.K % (8 * kStep) == 0;
+  if (p.K % kStep == 0 && (even || (p.K >= 40 * kStep && !(p.M <= 8 && p.N <= 4096)))) {
     if (p.M <= 16) return launch_lds<1, 1, 4>(p, s);
     if (p.M <= 32) return launch_lds<2, 1, 1>(p, s);
     // 32 weight rows per workgroup halve the activation re-reads, but up to N = 4096 they leave half the CUs

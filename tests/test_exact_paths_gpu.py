@@ -313,3 +313,20 @@ def test_k_split_exact(M, N, K, bias_dtype, fp16_out):
     torch.cuda.synchronize()
     _same_bits(y2, want, f"unsplit {M}x{N}x{K}")
 
+
+@pytest.mark.parametrize("M,N,K", [(1, 8192, 5248), (9, 1000, 5376), (16, 4096, 6784), (33, 2560, 5504), (48, 768, 11008), (64, 520, 13824),
+                                   (4, 4096, 11008), (20, 1024, 2560)])
+def test_weight_streaming_kernel_exact_on_k_loops_that_do_not_divide_among_its_waves(M, N, K):
+    """M <= 64 on narrow weights: the weight-streaming kernel deals whole K steps of 128 bytes to its eight waves.  With
+    K % 1024 != 0 (11008, 13824 and the like) the waves get unequal shares and the last batch is partly empty; the last
+    two cases stay on the register-direct form of the kernel (few rows on few weight rows; a short K)."""
+    from mslk_amd import _lib
+    name = _lib.lib().mslk_amd_debug_dispatch_name(M, N, K, 2, 0, 0, 1).decode()
+    assert name.startswith("skinny_registers" if (M, K) in ((4, 11008), (20, 2560)) else "skinny_lds"), name
+    g = torch.Generator().manual_seed(M + N + K)
+    xi, wi, xs, ws = _ints(M, K, g), _ints(N, K, g), _pow2(M, g), _pow2(N, g)
+    bias = torch.randint(-4, 5, (N,), generator=g).float()
+    y = torch.ops.mslk.f8f8bf16_rowwise(xi.to(F8).to(DEV), wi.to(F8).to(DEV), xs.to(DEV), ws.to(DEV), bias=bias.bfloat16().to(DEV))
+    torch.cuda.synchronize()
+    _same_bits(y, _want(xi, wi, xs, ws, bias), f"{M}x{N}x{K}")
+
