@@ -275,6 +275,68 @@ def _vendor_sweep(api):
                       "min_ratio": round(ratios[0], 3), "max_ratio": round(ratios[-1], 3)}))
 
 
+def _vendor_random(api, seed, cases):
+    """`--only vendor-random --seed S --cases N`: as `--only vendor`, on N shapes drawn with seed S -- M log-uniform in
+    1 ... 23000 (40 %: a batch size from a fixed list), N and K from the dimensions of common models, capped at 2^41
+    multiply-adds.  Prints one line per shape with the kernel the dispatch picks, then the shapes this library is behind on."""
+    import random
+    import torch
+    import mslk_amd
+    dev = "cuda:0"
+    rnd = random.Random(seed)
+    g = torch.Generator(device=dev).manual_seed(7)
+
+    def q(r, c, s=1.0):
+        return mslk_amd.quantize_fp8_row((torch.randn(r, c, device=dev, generator=g) * s).bfloat16(), use_triton=False)
+
+    def best_us(fn):
+        for i in range(6):
+            fn(i)
+        torch.cuda.synchronize()
+        return min(_events_ms(fn, 30) for _ in range(3)) * 1e3
+
+    res = []
+    for _ in range(cases):
+        N = rnd.choice([512, 1024, 1536, 2048, 2560, 3072, 3584, 4096, 5120, 6144, 7168, 8192, 11008, 12288, 13824, 14336, 16384,
+                        22016, 24576, 32768])
+        K = rnd.choice([512, 1024, 2048, 2560, 3072, 4096, 5120, 6144, 7168, 8192, 11008, 13824, 14336, 16384])
+        M = int(2 ** rnd.uniform(0, 14.5))
+        if rnd.random() < 0.4:
+            M = rnd.choice([8, 32, 48, 96, 192, 320, 768, 1536, 3072, 6144, 12288])
+        while M * N * K > 2 ** 41:
+            M //= 2
+        M = max(M, 1)
+        nsets = max(2, min(6, (400 << 20) // (N * K)))
+        ws = [q(N, K, 0.02) for _ in range(nsets)]
+        xs = [q(M, K) for _ in range(nsets)]
+        y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+
+        def ours(i):
+            j = i % nsets
+            api.gemm(xs[j][0], ws[j][0], xs[j][1], ws[j][1], y)
+
+        def vendor(i):
+            j = i % nsets
+            torch._scaled_mm(xs[j][0], ws[j][0].t(), scale_a=xs[j][1][:, None], scale_b=ws[j][1][None, :], out_dtype=torch.bfloat16)
+
+        try:
+            vendor(0)
+            tv = best_us(vendor)
+        except Exception:   # the vendor library may not take the shape
+            tv = float("nan")
+        to = best_us(ours)
+        name = api.L.mslk_amd_debug_dispatch_name(M, N, K, 0, 0, 0, 1).decode()
+        print(f"M={M:6d} N={N:6d} K={K:6d}: ours {to:8.1f} us  vendor {tv:8.1f} us  vendor/ours {tv / to:5.2f}  "
+              f"{2.0 * M * N * K / to / 1e9:5.2f} PFLOP/s  {name}", flush=True)
+        res.append((tv / to, M, N, K))
+        del ws, xs, y
+    ok = [r for r in res if r[0] == r[0]]
+    ok.sort()
+    print(json.dumps({"seed": seed, "shapes": len(res), "ours_faster": sum(1 for r in ok if r[0] >= 1.0),
+                      "median_ratio": ok[len(ok) // 2][0] if ok else None,
+                      "behind": [{"M": M, "N": N, "K": K, "vendor_over_ours": round(r, 3)} for (r, M, N, K) in ok if r < 1.0]}))
+
+
 def _ceilings(api):
     """`--only ceilings`: what this GPU sustains on the two resources the roofline fractions are priced against, from
     kernels that live in the library (mslk_amd_debug_stream_read / mslk_amd_debug_mfma_loop): a pure read of HBM-resident
@@ -368,7 +430,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", default="",
-                    help="helper: run only this piece (gemm|gemm-timed|power|phases|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|ceilings) and exit")
+                    help="helper: run only this piece (gemm|gemm-timed|power|phases|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|vendor-random|ceilings) and exit")
+    ap.add_argument("--seed", type=int, default=1, help="--only vendor-random: seed of the shape draw")
+    ap.add_argument("--cases", type=int, default=80, help="--only vendor-random: number of shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (no collectives or sharding in the path); "
@@ -385,6 +449,9 @@ def main():
     extras = {}
     if args.only == "vendor":
         _vendor_sweep(api)
+        return
+    if args.only == "vendor-random":
+        _vendor_random(api, args.seed, args.cases)
         return
     if args.only == "ceilings":
         _ceilings(api)
