@@ -205,10 +205,10 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // 46.4 -> 39.0 us; M = 12, N = 28672, K = 8192 45.3 -> 39.8 us), down to M <= 16, where the 32 x 32 tiles hold up to
   // N = 16384 (N = 14336, K = 8192: 22.8 against 23.4 us).
   if (p.M <= 64 && p.N >= kShortTileMinN) {
-    if (p.M <= 32 && p.N <= (p.M <= 16 ? 16384 : 8192)) return launch_tiled_shape<TileShape<32, 32, 2, 1, 8>, false, 2>(p, s);
+    if (p.M <= 32 && p.N <= (p.M <= 16 ? 16384 : 8192)) return launch_dense_small_tile(kTile32x32, p, s);
     if (p.M > 32 ? p.N <= 8192 : (p.N > 16384 && p.N < 24576))   // M = 9, N = 22016, K = 8192: 36.8 against 38.9 us on 64 x 64 tiles
-      return launch_tiled_shape<TileShape<64, 32, 4, 1, 6>, false, 2>(p, s);
-    return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false, 1>(p, s);
+      return launch_dense_small_tile(kTile64x32, p, s);
+    return launch_dense_small_tile(kTile64x64, p, s);
   }
   if (big_tiles > cus) return launch_persistent_shape<TileShape<256, 256>, false>(p, cus, s);
   // 128 x 256 tiles (wave tile 64 x 128, three ring buffers, one workgroup per CU) when they cover 160 ... 256 CUs in
@@ -222,7 +222,7 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
   // M = 768, N = 6144, K = 7168: 47.5 -> 40.6; M = 768, N = K = 8192: 54.6 -> 49.0).
   if (small_tiles > cus && big_tiles <= cus / 2) {
     const int64_t tiles19 = (int64_t)((p.M + 191) / 192) * ((p.N + 127) / 128);
-    if (tiles19 <= cus) return launch_tiled_shape<TileShape<192, 128, 2, 2, 3>, false>(p, s);
+    if (tiles19 <= cus) return launch_dense_small_tile(kTile192x128, p, s);
   }
   {
     const int64_t rows128 = (p.M + 127) / 128;
@@ -249,12 +249,18 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
     const int64_t tiles64 = (int64_t)((p.M + 63) / 64) * ((p.N + 63) / 64);
     const int64_t rows128 = (p.M + 127) / 128;
     const int64_t tiles128 = small_tiles <= cus / 4 ? rows128 * ((p.N + 31) / 32) : small_tiles <= cus / 2 ? rows128 * ((p.N + 63) / 64) : small_tiles;
-    if (tiles64 <= cus && tiles64 >= tiles128) return launch_tiled_shape<TileShape<64, 64, 4, 1, 5>, false, 1>(p, s);
+    if (tiles64 <= cus && tiles64 >= tiles128) return launch_dense_small_tile(kTile64x64, p, s);
   }
-  if (small_tiles <= cus / 4 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, false, 1>(p, s);
-  if (small_tiles <= cus / 2 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, false, 1>(p, s);
-  if (small_tiles <= cus) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, false, 1>(p, s);
-  return launch_tiled_shape<TileShape<128, 128>, false>(p, s);
+  if (small_tiles <= cus / 4 && p.N >= 64) return launch_dense_small_tile(kTile128x32, p, s);
+  if (small_tiles <= cus / 2 && p.N >= 128) return launch_dense_small_tile(kTile128x64, p, s);
+  if (small_tiles <= cus) {
+    // 96 x 128 tiles (wave tile 48 x 64, ring of five) where they fit one per CU as well: never more work per tile, and
+    // more tiles wherever M is not close under a multiple of 128 (M = 384, N = K = 8192: 192 -> 256 tiles, 39.5 -> 35.6 us;
+    // M = 320, N = 6144, K = 13824: 144 -> 192 tiles, 61.5 -> 53.3 us; M = 192, N = 14336: the same 224 tiles, 21.8 us both)
+    if ((int64_t)((p.M + 95) / 96) * ((p.N + 127) / 128) <= cus) return launch_dense_small_tile(kTile96x128, p, s);
+    return launch_dense_small_tile(kTile128x128Ring, p, s);
+  }
+  return launch_dense_small_tile(kTile128x128, p, s);
 }
 
 hipError_t launch_generic(const GemmProblem& p, hipStream_t s) {

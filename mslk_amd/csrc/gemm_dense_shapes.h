@@ -1,7 +1,7 @@
 // Tile-shape kernels of the dense f8f8bf16_rowwise GEMM and their launchers: one tile per workgroup and the persistent
 // form, each for row-major and for pre-shuffled weights.  Included by the translation units that instantiate them
-// (gemm_dense.hip: row-major weights; gemm_dense_preshuffled.hip: pre-shuffled weights), so that the two sets compile
-// side by side.
+// (gemm_dense.hip: the large shapes on row-major weights; gemm_dense_small.hip: the small ones; gemm_dense_preshuffled.hip:
+// pre-shuffled weights), so that the sets compile side by side.
 #pragma once
 #include "gemm_tile.h"
 #include "kernels.h"

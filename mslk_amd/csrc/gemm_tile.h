@@ -358,7 +358,7 @@ struct GemmTile {
     constexpr int NDMA = (ND + HALF - 1) / HALF;                      // DMA loads per MFMA group (first half only)
     constexpr int PER_SLOT = (NDMA + TS::FM - 1) / TS::FM;            // 1 unless the tile has few MFMAs per group
     constexpr int SLOTS = PER_SLOT > 0 ? (NDMA + PER_SLOT - 1) / PER_SLOT : 0;   // MFMA slots of a group that carry loads
-    constexpr bool SPREAD = PER_SLOT <= 1 && ND <= GD * TS::FM;
+    constexpr bool SPREAD = (PER_SLOT <= 1 || ND % HALF != 0) && ND <= GD * TS::FM;   // also: a load count the halves cannot share evenly
     static_assert(SPREAD || ND % HALF == 0, "DMA loads spread evenly over the first half");
     const FragOff fo = frag_off();
     const char* b_tile = b_tile_of(b_cur);

@@ -82,6 +82,14 @@ int device_compute_units();
 // Shape classes; each returns hipErrorInvalidValue when the shape is outside what it supports.
 bool dense_tiled_supports(const GemmProblem& p);
 hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s);
+// The tile shapes below 128 x 256 on row-major weights (gemm_dense_small.hip), launched by name.
+enum DenseSmallTile : int {
+  kTile32x32, kTile64x32, kTile64x64, kTile128x32, kTile128x64, kTile96x128,
+  kTile128x128Ring,   // five ring buffers, one workgroup per CU
+  kTile128x128,       // two-plus-three buffers, two workgroups per CU
+  kTile192x128,
+};
+hipError_t launch_dense_small_tile(int shape, const GemmProblem& p, hipStream_t s);
 // Its branch for pre-shuffled weights (a translation unit of its own); cus: device_compute_units().
 hipError_t launch_dense_tiled_preshuffled(const GemmProblem& p, int cus, hipStream_t s);
 // K-split form for shapes with few output tiles and a long K (gemm_splitk.hip): `slices` workgroups per tile of edge
@@ -150,5 +158,8 @@ struct DeviceGroups {
   int unaligned;        // set by the launcher: operands need the scalar tile path
 };
 hipError_t launch_device_groups(const DeviceGroups& p, int layout, hipStream_t s);
+// Its layouts outside gemm_grouped.hip (translation units of their own); p.unaligned already set.
+hipError_t launch_device_groups_layouts(const DeviceGroups& p, int layout, hipStream_t s);
+hipError_t launch_device_groups_uniform(const DeviceGroups& p, hipStream_t s);
 
 }  // namespace mslk_amd

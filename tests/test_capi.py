@@ -186,6 +186,7 @@ DISPATCH_TABLE = [
     ((128, 4096, 14336, 2, 1, 0, 1), "splitk_partial<64,64,waves=4x1,ring=5> slices=2 + splitk_reduce"),
     ((128, 4096, 4096, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=128"),                          # K too short to split                      # 128 x 128 tiles would need two passes
     ((512, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,128,waves=2x2,ring=5> tiles=256"),
+    ((384, 8192, 8192, 0, 0, 0, 1), "dense_tiled<96,128,waves=2x2,ring=5> tiles=256"),                        # 96-row tiles still fit one per CU: 256 instead of 192 tiles
     ((256, 8192, 8192, 0, 0, 0, 1), "dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
     ((128, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> tiles=256"),
     ((64, 10240, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> weights streamed tiles=160"),         # one row of tiles: non-temporal weight loads

@@ -269,10 +269,11 @@ def test_preshuffled_tiles_exact(M, N, K, fp16_out):
 
 @pytest.mark.parametrize("M,N,K", [(1024, 8192, 384), (2048, 4096, 272), (96, 8192, 512), (128, 4096, 400), (40, 8192, 1040),
                                    (24, 12288, 256), (16, 12288, 256), (24, 20480, 384), (64, 16384, 384), (1536, 6144, 144),
+                                   (300, 8192, 528), (280, 8000, 400), (384, 8192, 256),        # 96 x 128 tiles, ring of five
                                    (1000, 5000, 528), (768, 7168, 256), (960, 6144, 128),       # 192 x 128 tiles, ring of three
                                    (1536, 6144, 2064), (1500, 6100, 2048)])                      # 192 x 256 tiles, two-plus-three buffers
 def test_ring_and_short_tiles_exact(M, N, K):
-    """The symmetric-ring tile shapes (128 x 256, 192 x 128, 128 x 128, 128 x 64, 128 x 32, 64 x 64, 64 x 32, 32 x 32): their
+    """The symmetric-ring tile shapes (128 x 256, 192 x 128, 128 x 128, 96 x 128, 128 x 64, 128 x 32, 64 x 64, 64 x 32, 32 x 32): their
     barrier waits on a load count that covers several steps in flight; and the 192 x 256 tiles (six m fragments per wave on
     the two-plus-three buffers).  Ragged last tiles along M and N, K loops shorter than the ring, K tails."""
     g = torch.Generator().manual_seed(M + N + K)
