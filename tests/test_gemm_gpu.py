@@ -268,7 +268,8 @@ def test_k_not_a_multiple_of_16_runs_on_padded_copies(M, N, K):
         assert torch.equal(y_plain.view(torch.int16), y_small.view(torch.int16))
 
 
-@pytest.mark.parametrize("M,N,K", [(512, 1024, 512), (16, 1024, 1024), (4352, 4352, 128), (16, 8192, 256), (64, 8192, 256)])
+@pytest.mark.parametrize("M,N,K", [(512, 1024, 512), (16, 1024, 1024), (4352, 4352, 128), (16, 8192, 256), (64, 8192, 256),
+                                   (128, 1024, 8192)])   # the last one is split along K: two launches and a workspace from the graph's pool
 def test_hip_graph_capture_and_replay(M, N, K):
     """The reference tests capture + replay (test/gemm/gemm_test.py:440-447); replay several times with
     eager work in between and compare every replay with the eager result."""
