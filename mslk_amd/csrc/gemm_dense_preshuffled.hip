@@ -18,7 +18,10 @@ hipError_t launch_dense_tiled_preshuffled(const GemmProblem& p, int cus, hipStre
   if (big_tiles >= cus * 3 / 4) return launch_tiled_shape<TileShape<256, 256>, true>(p, s);
   if (small_tiles <= cus / 4 && p.N >= 64) return launch_tiled_shape<TileShape<128, 32, 4, 1, 8>, true>(p, s);
   if (small_tiles <= cus / 2 && p.N >= 128) return launch_tiled_shape<TileShape<128, 64, 4, 1, 6>, true>(p, s);
-  if (small_tiles <= cus) return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
+  if (small_tiles <= cus) {   // 96-row tiles where they fit one per CU as well: more tiles, never more work per tile
+    if ((int64_t)((p.M + 95) / 96) * ((p.N + 127) / 128) <= cus) return launch_tiled_shape<TileShape<96, 128, 2, 2, 5>, true>(p, s);
+    return launch_tiled_shape<TileShape<128, 128, 2, 2, 5>, true>(p, s);
+  }
   if (big_tiles <= cus / 2 && (int64_t)((p.M + 191) / 192) * ((p.N + 127) / 128) <= cus)
     return launch_tiled_shape<TileShape<192, 128, 2, 2, 3>, true>(p, s);
   return launch_tiled_shape<TileShape<128, 128>, true>(p, s);
