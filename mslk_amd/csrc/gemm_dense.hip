@@ -171,7 +171,10 @@ hipError_t launch_dense_tiled(const GemmProblem& p, hipStream_t s) {
       const int64_t passes = (tiles + wgs - 1) / wgs;
       const int64_t last = tiles - (passes - 1) * wgs;           // tiles of the last pass
       const int64_t rows1 = ((passes - 1) * wgs / tiles_n) * 256;   // rows whose tiles fit the full passes
-      if (last * 2 <= wgs && rows1 > 0 && rows1 < p.M) {
+      // ... and up to three quarters full when the remaining rows fit one pass of 192 x 256 tiles: a quarter less work
+      // per tile than the pass of 256 x 256 tiles they replace
+      const int64_t rest192 = (p.M - rows1 + 191) / 192 * tiles_n;
+      if ((last * 2 <= wgs || (last * 4 <= wgs * 3 && rest192 <= wgs && p.K >= 2048)) && rows1 > 0 && rows1 < p.M) {
         GemmProblem a = p, b = p;
         a.M = (int)rows1;
         b.M = p.M - (int)rows1;

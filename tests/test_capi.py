@@ -176,6 +176,8 @@ DISPATCH_TABLE = [
     ((3, 1000, 272, 0, 0, 0, 1), "skinny_registers<m_frags=1,n_frags=1,steps=8> workgroups=63"),              # K % 1024 != 0
     ((8192, 8192, 8192, 0, 0, 0, 1), "dense_persistent<256,256> tiles=1024 workgroups=256"),
     ((2304, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256 + dense_tiled<128,64,waves=4x1,ring=6> tiles=256"),
+    ((3328, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=256 + dense_tiled<192,256,waves=2x2,ring=0> tiles=224"),   # last pass 5/8 full: its rows on 192-row tiles
+    ((3840, 8192, 8192, 0, 0, 0, 1), "dense_persistent<256,256> tiles=480 workgroups=256"),                  # 7/8 full: one persistent launch
     ((2048, 4096, 4096, 0, 0, 0, 1), "dense_tiled<128,256,waves=2x2,ring=3> tiles=256"),
     ((1536, 6144, 8192, 0, 0, 0, 1), "dense_tiled<192,256,waves=2x2,ring=0> tiles=192"),                     # 144 tiles of 256 x 256: 192-row tiles still fit one per CU
     ((1728, 8192, 8192, 0, 0, 0, 1), "dense_tiled<256,256,waves=2x2,ring=0> tiles=224"),                     # ... and here they do not

@@ -268,6 +268,17 @@ def test_preshuffled_tiles_exact(M, N, K, fp16_out):
         _same_bits(y, _want(xi, wi, xs, ws, b, fp16_out), f"pre-shuffled {M}x{N}x{K} bias={'yes' if b is not None else 'no'}")
 
 
+def test_rows_of_a_partly_filled_last_pass_go_to_a_second_launch_exact():
+    """416 tiles of 256 x 256 on 256 CUs: the 2048 rows of the first pass and the 1280 rows behind them are two launches
+    (256 x 256 tiles, then 192 x 256 tiles); the seam between them must not show."""
+    M, N, K = 3328, 8192, 2048
+    g = torch.Generator().manual_seed(M + N + K)
+    xi, wi, xs, ws = _ints(M, K, g), _ints(N, K, g), _pow2(M, g), _pow2(N, g)
+    y = torch.ops.mslk.f8f8bf16_rowwise(xi.to(F8).to(DEV), wi.to(F8).to(DEV), xs.to(DEV), ws.to(DEV))
+    torch.cuda.synchronize()
+    _same_bits(y, _want(xi, wi, xs, ws), f"{M}x{N}x{K}")
+
+
 @pytest.mark.parametrize("M,N,K", [(1024, 8192, 384), (2048, 4096, 272), (96, 8192, 512), (128, 4096, 400), (40, 8192, 1040),
                                    (24, 12288, 256), (16, 12288, 256), (24, 20480, 384), (64, 16384, 384), (1536, 6144, 144),
                                    (300, 8192, 528), (280, 8000, 400), (384, 8192, 256),        # 96 x 128 tiles, ring of five
