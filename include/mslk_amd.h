@@ -175,7 +175,7 @@ size_t mslk_amd_static_scratch_bytes(void);
  * Decode fast path: row-wise quantization of the activations AND the GEMM in one launch.  Replaces the pair
  * quantize_fp8_row(x) -> f8f8bf16_rowwise(xq, wq, x_scale, w_scale) that callers of the reference issue for every
  * decode step (reference: bench/gemm/gemm_ops.py:593-673; mslk/moe/layers.py:1096,1123), for the shapes where the first
- * launch costs about as much as the work: 1 <= M <= 4, K % 1024 == 0 (mslk_amd_quantize_f8f8bf16_rowwise_supported).
+ * launch costs about as much as the work: 1 <= M <= 4, K >= 1024, K % 128 == 0 (mslk_amd_quantize_f8f8bf16_rowwise_supported).
  *   x    [M, K] bf16 (x_dtype must be MSLK_AMD_DTYPE_BF16), row stride x_row_stride elements (a multiple of 8), 16-byte aligned
  *   wq, w_scale, bias, y   as mslk_amd_f8f8bf16_rowwise
  *   xq_out [M, K] e4m3fn, x_scale_out [M] fp32: optional (NULL to skip); they receive the codes and scales the kernel

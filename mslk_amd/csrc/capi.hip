@@ -267,7 +267,7 @@ int mslk_amd_f8f8bf16_rowwise_static_scratch(const void* xq, const void* wq, con
 }
 
 int mslk_amd_quantize_f8f8bf16_rowwise_supported(int64_t M, int64_t N, int64_t K) {
-  return M >= 1 && M <= 4 && N >= 1 && N <= kIntMax && K >= 1024 && K % 1024 == 0 && K <= (int64_t(1) << 25);
+  return M >= 1 && M <= 4 && N >= 1 && N <= kIntMax && K >= 1024 && K % 128 == 0 && K <= (int64_t(1) << 25);
 }
 
 int mslk_amd_quantize_f8f8bf16_rowwise(const void* x, int x_dtype, int64_t x_row_stride, const void* wq, const float* w_scale,

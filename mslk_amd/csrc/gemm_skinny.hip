@@ -525,7 +525,7 @@ __global__ __launch_bounds__(512) void skinny_fused_quant_kernel(GemmProblem p, 
   char* cbuf = xbuf + WBYTES;
   const char* xfrag = cbuf + (i < M ? i : M - 1) * 128 + g * 16;   // fragment rows beyond M repeat the last row; never stored
 
-  // 2. weight stream; K % (8 * 128) == 0: every wave owns KT / 8 complete steps
+  // 2. weight stream: whole K steps, dealt to the eight waves in batches of U (the last batch may be partly empty)
   v4f acc = v4f{0.f, 0.f, 0.f, 0.f};
   const int KT = K / kStep;
   for (int kt0 = wave; kt0 < KT; kt0 += kWaves * U) {
@@ -589,7 +589,7 @@ __global__ __launch_bounds__(512) void skinny_fused_quant_kernel(GemmProblem p, 
 }  // namespace
 
 bool skinny_fused_quant_supports(const GemmProblem& p, const void* x, int64_t x_stride) {
-  return p.M >= 1 && p.M <= kFusedMaxM && p.N >= 1 && p.K >= 1024 && p.K % (8 * kStep) == 0 &&
+  return p.M >= 1 && p.M <= kFusedMaxM && p.N >= 1 && p.K >= 1024 && p.K % kStep == 0 &&
          (int64_t)64 * p.K < (int64_t(1) << 32) && !p.w_preshuffled && x_stride >= p.K && x_stride % 8 == 0 &&
          reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(p.wq) % 16 == 0;
 }

@@ -161,7 +161,7 @@ def f8f8bf16_rowwise_out(XQ, WQ, x_scale, w_scale, output, bias=None, use_fast_a
 def quantize_f8f8bf16_rowwise(X, WQ, w_scale, bias=None):
     """bf16 activations in, bf16 out: `quantize_fp8_row(X, use_triton=False)` followed by `f8f8bf16_rowwise`, returning
     (Y, XQ, x_scale) -- the pair every decode step of a caller of the reference issues (bench/gemm/gemm_ops.py:593-673).
-    For 1 <= M <= 4 rows of bf16 with K % 1024 == 0 it is ONE launch (every workgroup quantizes the rows itself; XQ and
+    For 1 <= M <= 4 rows of bf16 with K % 128 == 0 (K >= 1024) it is ONE launch (every workgroup quantizes the rows itself; XQ and
     x_scale are the bits the stand-alone quantizer returns); other shapes run the two kernels."""
     _check(WQ.dtype == FP8_DTYPE, f"WQ must be {FP8_DTYPE} on gfx950, got {WQ.dtype}")
     _check(w_scale.dtype == torch.float32, "Scales must be float32.")

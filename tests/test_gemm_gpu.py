@@ -572,6 +572,7 @@ def test_matches_the_model_level_fake_quant_statement(M, N, K):
 @pytest.mark.parametrize("M,N,K,bias_dtype", [(1, 512, 1024, None), (3, 1000, 2048, torch.bfloat16), (4, 8200, 5120, torch.float32),
                                               (2, 48, 3072, None), (4, 16, 8192, torch.bfloat16), (2, 4096, 14336, None),
                                               (1, 520, 15360, None), (3, 300, 16384, None),
+                                              (2, 4096, 11008, None), (4, 1000, 13824, torch.bfloat16), (1, 264, 1152, None),   # K steps that do not divide among the waves
                                               (7, 520, 2048, None), (4, 300, 1040, torch.bfloat16)])   # the last two: two launches
 def test_quantize_fused_into_the_decode_gemm(M, N, K, bias_dtype):
     """quantize_f8f8bf16_rowwise: codes and scales are the stand-alone quantizer's bits (checked against the oracle),
