@@ -28,7 +28,7 @@ int check_hip(hipError_t e, const char* what) {
 
 constexpr int64_t kIntMax = 2147483647;
 
-// Device memory for the padded operand copies of mslk_amd_f8f8bf16_rowwise_static_scratch: part of the code object, so
+// Device memory for the padded operand copies (or the fp32 sums of a K split) of mslk_amd_f8f8bf16_rowwise_static_scratch: part of the code object, so
 // every GPU the library runs on holds its own copy from module load until the process ends.  In host code the name
 // below is only a handle for hipGetSymbolAddress; kernels and copies get the per-device address it returns.
 constexpr size_t kScratchBytes = MSLK_AMD_STATIC_SCRATCH_BYTES;
