@@ -60,6 +60,20 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
     assert L.mslk_amd_quantize_fp8_row(None, 0, 0, 16, 16, None, 16, None, None, None) == 0
 
 
+@pytest.mark.parametrize("M,N,K,slices", [
+    (64, 512, 14336, 0), (65, 512, 14336, 8),            # more than 64 rows only: below, the weight-streaming kernel covers the CUs
+    (128, 512, 8192, 8), (128, 512, 6144, 6),            # as many slices as fill the CUs once, at least eight K steps each
+    (128, 512, 4096, 0),                                 # K too short for two launches to pay
+    (128, 4096, 8192, 2), (128, 4096, 6144, 0),          # half the CUs covered: from K = 8192 on
+    (128, 4160, 8192, 0), (512, 1024, 8192, 2), (512, 1088, 8192, 0), (1024, 512, 16384, 2), (1025, 512, 16384, 0),   # at most 128 tiles of 64 x 64
+    (96, 2048, 8192, 4), (300, 518, 6160, 5), (128, 63, 8192, 0),
+])
+def test_k_split_plan_is_pinned(M, N, K, slices):
+    """mslk_amd_f8f8bf16_rowwise_workspace_bytes is the plan: slices * M * N floats for a shape the library splits along K
+    (on a whole MI355X, which is also what the library assumes when no device can be queried), 0 otherwise."""
+    assert _lib.lib().mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K) == slices * M * N * 4
+
+
 def test_ops_registered_with_reference_schemas():
     s = str(torch.ops.mslk.f8f8bf16_rowwise.default._schema)
     assert s == ("mslk::f8f8bf16_rowwise(Tensor XQ, Tensor WQ, Tensor x_scale, Tensor w_scale, "
