@@ -337,6 +337,54 @@ def _vendor_random(api, seed, cases):
                       "behind": [{"M": M, "N": N, "K": K, "vendor_over_ours": round(r, 3)} for (r, M, N, K) in ok if r < 1.0]}))
 
 
+def _ksplit(api):
+    """`--only ksplit`: shapes with few output tiles and a long K, timed with the workspace the library asks for (K split:
+    two launches) and without it (the ordinary kernels), same operands, rotating weight sets.  One line per shape."""
+    import torch
+    import mslk_amd
+    dev = "cuda:0"
+    L = api.L
+    g = torch.Generator(device=dev).manual_seed(3)
+
+    def q(r, c, s=1.0):
+        return mslk_amd.quantize_fp8_row((torch.randn(r, c, device=dev, generator=g) * s).bfloat16(), use_triton=False)
+
+    rows = []
+    for K in (6144, 8192, 14336):
+        for N in (512, 1024, 2048, 4096):
+            nsets = max(2, min(8, (300 << 20) // (N * K)))
+            ws = [q(N, K, 0.02) for _ in range(nsets)]
+            for M in (64, 96, 128, 256, 512):
+                need = L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+                xq, xs = q(M, K)
+                y = torch.empty(M, N, dtype=torch.bfloat16, device=dev)
+                wsp = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+
+                def run(with_workspace):
+                    def step(i):
+                        w, sc = ws[i % nsets]
+                        api.check(L.mslk_amd_f8f8bf16_rowwise(xq.data_ptr(), w.data_ptr(), xs.data_ptr(), sc.data_ptr(), None, 0, y.data_ptr(),
+                                                              M, N, K, wsp.data_ptr() if with_workspace else None,
+                                                              need if with_workspace else 0, api.stream))
+                    for i in range(5):
+                        step(i)
+                    torch.cuda.synchronize()
+                    return min(_median_events_ms(step, 40) for _ in range(2)) * 1e3
+
+                unsplit = run(False)
+                split = run(True) if need else None
+                name = L.mslk_amd_debug_dispatch_name(M, N, K, 0, 0, 0, 1).decode()
+                rows.append({"M": M, "N": N, "K": K, "unsplit_us": round(unsplit, 2), "with_workspace_us": None if split is None else round(split, 2),
+                             "slices": need // (M * N * 4), "dispatch": name})
+                print(f"M={M:4d} N={N:5d} K={K:6d}: unsplit {unsplit:6.1f} us | " +
+                      (f"K split in {need // (M * N * 4)} slices {split:6.1f} us ({unsplit / split:4.2f}x)" if need else "not split"), flush=True)
+            del ws
+    done = [r for r in rows if r["with_workspace_us"]]
+    print(json.dumps({"shapes": len(rows), "split": len(done),
+                      "slower_than_unsplit_by_more_than_2_percent": sum(1 for r in done if r["with_workspace_us"] > 1.02 * r["unsplit_us"]),
+                      "best_ratio": max(r["unsplit_us"] / r["with_workspace_us"] for r in done) if done else None}))
+
+
 def _ceilings(api):
     """`--only ceilings`: what this GPU sustains on the two resources the roofline fractions are priced against, from
     kernels that live in the library (mslk_amd_debug_stream_read / mslk_amd_debug_mfma_loop): a pure read of HBM-resident
@@ -430,7 +478,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--only", default="",
-                    help="helper: run only this piece (gemm|gemm-timed|power|phases|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|vendor-random|ceilings) and exit")
+                    help="helper: run only this piece (gemm|gemm-timed|power|phases|quantize|decode|decode-eager|decode-graph|cfg2|grouped|traffic|vendor|vendor-random|ksplit|ceilings) and exit")
     ap.add_argument("--seed", type=int, default=1, help="--only vendor-random: seed of the shape draw")
     ap.add_argument("--cases", type=int, default=80, help="--only vendor-random: number of shapes")
     args = ap.parse_args()
@@ -449,6 +497,9 @@ def main():
     extras = {}
     if args.only == "vendor":
         _vendor_sweep(api)
+        return
+    if args.only == "ksplit":
+        _ksplit(api)
         return
     if args.only == "vendor-random":
         _vendor_random(api, args.seed, args.cases)
