@@ -137,7 +137,8 @@ int mslk_amd_gather_scale_quant_dense_tokens(const void* x, int x_dtype, int64_t
  *     fp8_rowwise_common.h:109-110 `GemmSpecialization::MNKPadding`).  An operand base pointer that is not 16-byte aligned
  *     is handled the same way if the workspace holds (M + N) * round_up(K, 16) bytes.  Without a workspace (null or too
  *     small) such operands still give the same results through a scalar kernel that is orders of magnitude slower.
- *   - few output tiles and a long K (64 < M, at most 128 tiles of 64 x 64 on a whole MI355X, K >= 6144 ... 8192; the
+ *   - few output tiles and a long K (64 < M, or 32 < M with K >= 12288; at most 128 tiles of 64 x 64 on a whole MI355X,
+ *     K >= 6144 ... 8192; the
  *     reference's instances for such shapes split K as well, fp8_rowwise_common.h:168-204 `KBatch`): the call cuts K into
  *     2 ... 8 slices, whose fp32 sums go into the workspace (slices * M * N floats), and a second launch adds them and
  *     applies scales, bias and the conversion -- two to three times faster where the unsplit kernels would leave most

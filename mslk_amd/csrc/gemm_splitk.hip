@@ -106,13 +106,14 @@ hipError_t launch_reduce(const GemmProblem& p, const float* part, int slices, hi
 // The plan for a shape: number of K slices on 64 x 64 tiles; 1 means "do not split".  Measured on M = 16 ... 512,
 // N = 512 ... 8192, K = 4096 / 8192 / 14336 against the unsplit dispatch: the two launches cost about 10 us, so a split
 // pays only where the unsplit launch is a long K loop on few CUs -- more than 64 rows (below that the weight-streaming
-// kernel and the short tiles already cover the CUs), at most half as many 64 x 64 tiles as CUs, K from 8192 on (6144
+// kernel and the short tiles already cover the CUs; 33 ... 64 rows gain only from K = 12288 on: M = 64, N = 4096, K = 14336
+// 22.4 -> 19.1 us, but K = 8192 10.2 -> 12.7), at most half as many 64 x 64 tiles as CUs, K from 8192 on (6144
 // when the tiles cover at most a quarter of the CUs); then as many slices as fill the CUs once, at most eight, each at
 // least eight K steps long.  M = 128, N = 512, K = 14336: 37.8 -> 12.4 us; M = 96, N = 2048, K = 8192: 15.8 -> 11.9;
 // M = 128, N = 4096, K = 14336: 34.2 -> 24.8; 128 x 128 tiles in slices were slower than these on every shape.
 SplitKPlan splitk_plan(int64_t M, int64_t N, int64_t K, int cus) {
   SplitKPlan plan{64, 1};
-  if (M <= 64 || N < 64 || K < 6144 || K % 16 != 0) return plan;
+  if (M <= 32 || (M <= 64 && K < 12288) || N < 64 || K < 6144 || K % 16 != 0) return plan;
   const int64_t steps = K / kBK;
   const int64_t tiles = ((M + 63) / 64) * ((N + 63) / 64);
   if (tiles > cus / 2 || (K < 8192 && tiles > cus / 4)) return plan;   // (two slices on up to 3/4 of the CUs at K >= 12288: 3 - 17 % slower)

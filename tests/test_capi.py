@@ -30,7 +30,7 @@ def test_library_exports_every_declared_symbol():
     assert L.mslk_amd_version().decode().startswith("mslk_amd")
     assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(4096, 4096, 4096) == 0
     assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(128, 512, 14336) == 8 * 128 * 512 * 4      # eight K slices of fp32 sums
-    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(64, 512, 14336) == 0                      # M <= 64 is never split
+    assert L.mslk_amd_f8f8bf16_rowwise_workspace_bytes(64, 512, 8192) == 0                       # M <= 64 is not split below K = 12288
 
 
 def test_c_abi_rejects_bad_arguments_without_a_gpu():
@@ -61,7 +61,8 @@ def test_c_abi_rejects_bad_arguments_without_a_gpu():
 
 
 @pytest.mark.parametrize("M,N,K,slices", [
-    (64, 512, 14336, 0), (65, 512, 14336, 8),            # more than 64 rows only: below, the weight-streaming kernel covers the CUs
+    (64, 512, 8192, 0), (65, 512, 8192, 8),              # more than 64 rows: below, the weight-streaming kernel covers the CUs ...
+    (32, 512, 14336, 0), (33, 512, 14336, 8), (64, 4096, 12288, 4), (64, 4096, 11008, 0),   # ... except 33 - 64 rows at K >= 12288
     (128, 512, 8192, 8), (128, 512, 6144, 6),            # as many slices as fill the CUs once, at least eight K steps each
     (128, 512, 4096, 0),                                 # K too short for two launches to pay
     (128, 4096, 8192, 2), (128, 4096, 6144, 0),          # half the CUs covered: from K = 8192 on
@@ -181,7 +182,8 @@ DISPATCH_TABLE = [
     ((64, 8192, 8192, 0, 0, 0, 1), "dense_tiled<64,32,waves=4x1,ring=6> weights streamed tiles=256"),
     ((16, 8192, 8192, 0, 0, 1, 1), "skinny_lds<m_frags=1,n_frags=2,steps=2> preshuffled workgroups=256"),    # cfg3 on blocked weights
     ((64, 8192, 8192, 0, 0, 1, 1), "skinny_lds<m_frags=4,n_frags=2,steps=1> preshuffled workgroups=256"),
-    ((64, 4096, 14336, 0, 0, 0, 1), "skinny_lds<m_frags=4,n_frags=1,steps=1> workgroups=256"),
+    ((64, 4096, 14336, 0, 0, 0, 0), "skinny_lds<m_frags=4,n_frags=1,steps=1> workgroups=256"),
+    ((64, 4096, 14336, 0, 0, 0, 1), "splitk_partial<64,64,waves=4x1,ring=5> slices=4 + splitk_reduce"),       # 33 - 64 rows: split from K = 12288 on, given a workspace
     ((8, 8192, 8192, 0, 0, 0, 1), "skinny_lds<m_frags=1,n_frags=1,steps=4> workgroups=512"),                  # last M of the streaming kernel on wide weights
     ((9, 8192, 8192, 0, 0, 0, 1), "dense_tiled<32,32,waves=2x1,ring=8> weights streamed tiles=256"),
     ((32, 10240, 8192, 0, 0, 0, 1), "dense_tiled<64,64,waves=4x1,ring=5> weights streamed tiles=160"),        # M <= 32 on wider weights

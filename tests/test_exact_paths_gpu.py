@@ -298,7 +298,7 @@ def test_ring_and_short_tiles_exact(M, N, K):
 
 @pytest.mark.parametrize("fp16_out", [False, True])
 @pytest.mark.parametrize("bias_dtype", [None, torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("M,N,K", [(128, 512, 8192), (96, 2048, 8192), (300, 518, 6160), (65, 4096, 14336), (512, 1024, 8208)])
+@pytest.mark.parametrize("M,N,K", [(128, 512, 8192), (96, 2048, 8192), (300, 518, 6160), (65, 4096, 14336), (512, 1024, 8208), (40, 1000, 12304)])
 def test_k_split_exact(M, N, K, bias_dtype, fp16_out):
     """Few output tiles and a long K: with the workspace the library asks for, K is cut into slices whose fp32 sums a
     second launch adds, scales and converts (ragged rows and columns, a column count that rules out 16-byte accesses, a K
@@ -329,7 +329,7 @@ def test_k_split_exact(M, N, K, bias_dtype, fp16_out):
     _same_bits(y2, want, f"unsplit {M}x{N}x{K}")
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 8192, 5248), (9, 1000, 5376), (16, 4096, 6784), (33, 2560, 5504), (48, 768, 11008), (64, 520, 13824),
+@pytest.mark.parametrize("M,N,K", [(1, 8192, 5248), (9, 1000, 5376), (16, 4096, 6784), (33, 2560, 5504), (48, 768, 11008), (64, 520, 11264),
                                    (4, 4096, 11008), (20, 1024, 2560)])
 def test_weight_streaming_kernel_exact_on_k_loops_that_do_not_divide_among_its_waves(M, N, K):
     """M <= 64 on narrow weights: the weight-streaming kernel deals whole K steps of 128 bytes to its eight waves.  With
