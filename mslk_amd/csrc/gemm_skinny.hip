@@ -619,7 +619,10 @@ bool skinny_supports(const GemmProblem& p) {
 
 hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
   if (!skinny_supports(p)) return hipErrorInvalidValue;
-  if (p.w_preshuffled && p.K % (8 * kStep) == 0 && p.M > 4) {
+  // (K steps that do not divide among the eight waves, as below: from 40 steps on, except for at most 16 rows on at most
+  // 4096 weight rows -- M = 64, N = 8192, K = 13824: 35.6 -> 28.0 us; M = 8, N = 4096, K = 11008: 9.3 against 12.2 us)
+  if (p.w_preshuffled && p.K % kStep == 0 && p.M > 4 &&
+      (p.K % (8 * kStep) == 0 || (p.K >= 40 * kStep && !(p.M <= 16 && p.N <= 4096)))) {
     // weights straight into registers (contiguous KiB blocks), activations through LDS
     if (p.M <= 16) return launch_lds<1, 2, 2, true>(p, s);
     if (p.M <= 32) return launch_lds<2, 2, 1, true>(p, s);
