@@ -623,7 +623,14 @@ hipError_t launch_skinny(const GemmProblem& p, hipStream_t s) {
   // 4096 weight rows -- M = 64, N = 8192, K = 13824: 35.6 -> 28.0 us; M = 8, N = 4096, K = 11008: 9.3 against 12.2 us)
   if (p.w_preshuffled && p.K % kStep == 0 && p.M > 4 &&
       (p.K % (8 * kStep) == 0 || (p.K >= 40 * kStep && !(p.M <= 16 && p.N <= 4096)))) {
-    // weights straight into registers (contiguous KiB blocks), activations through LDS
+    // weights straight into registers (contiguous KiB blocks), activations through LDS; 16 weight rows per workgroup
+    // instead of 32 on narrow weights, which 32 would leave with fewer workgroups than CUs
+    if (p.N <= 4096) {
+      if (p.M <= 16) return launch_lds<1, 1, 4, true>(p, s);
+      if (p.M <= 32) return launch_lds<2, 1, 1, true>(p, s);
+      if (p.M <= 48) return launch_lds<3, 1, 1, true>(p, s);
+      return launch_lds<4, 1, 1, true>(p, s);
+    }
     if (p.M <= 16) return launch_lds<1, 2, 2, true>(p, s);
     if (p.M <= 32) return launch_lds<2, 2, 1, true>(p, s);
     if (p.M <= 48) return launch_lds<3, 2, 1, true>(p, s);

@@ -253,6 +253,7 @@ def test_batched_exact(G, M, N, K, bias_dtype):
     (200, 2048, 512),     # 128 x 64 / 64 x 64 narrow tiles
     (48, 4096, 1024),     # weight-streaming kernel on blocked weights
     (40, 2560, 5504), (20, 8192, 11008),   # ... on K steps that do not divide among its waves
+    (10, 2048, 2048), (30, 1024, 1024), (60, 4096, 1024), (60, 8192, 1024),   # 16 weight rows per workgroup up to N = 4096, 32 above
     (300, 8000, 448),     # 96 x 128 ring tiles
     (1000, 5008, 576),    # 192 x 128 tiles (ragged rows and columns; N % 16 == 0 and K % 64 == 0 as blocked weights need)
     (1500, 6096, 2112),   # 192 x 256 tiles
