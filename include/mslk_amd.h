@@ -211,6 +211,15 @@ int mslk_amd_f8f8f16_rowwise(const void* xq, const void* wq, const float* x_scal
 int mslk_amd_f8f8_rowwise_preshuffle(const void* xq, const void* wq_shuffled, const float* x_scale, const float* w_scale,
                                      const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M, int64_t N,
                                      int64_t K, void* stream);
+/*
+ * The same with the optional workspace of mslk_amd_f8f8bf16_rowwise (mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+ * bytes, 16-byte aligned): shapes with few output tiles and a long K are then split along K as on row-major weights.
+ * Without a workspace it is the entry point above.
+ */
+int mslk_amd_f8f8_rowwise_preshuffle_workspace(const void* xq, const void* wq_shuffled, const float* x_scale,
+                                               const float* w_scale, const void* bias, int bias_dtype, void* y, int y_dtype,
+                                               int64_t M, int64_t N, int64_t K, void* workspace, size_t workspace_bytes,
+                                               void* stream);
 
 /*
  * Weight re-layout for the entry point above: wq [G, N, K] row-major -> wq_shuffled, the blocked

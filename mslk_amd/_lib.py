@@ -42,6 +42,8 @@ SIGNATURES = {
                                          c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "mslk_amd_f8f8_rowwise_preshuffle": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
                                                  c_int64, c_int64, c_int64, c_void_p]),
+    "mslk_amd_f8f8_rowwise_preshuffle_workspace": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int,
+                                                           c_int64, c_int64, c_int64, c_void_p, c_size_t, c_void_p]),
     "mslk_amd_preshuffle_b": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
     "mslk_amd_f8f8bf16_rowwise_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
     "mslk_amd_f8f8bf16_rowwise_grouped": (c_int, [c_int, POINTER(c_void_p), POINTER(c_void_p), POINTER(c_void_p),

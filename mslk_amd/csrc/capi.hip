@@ -217,7 +217,7 @@ static int rowwise_impl(const char* op, int out_f16, int preshuffled, const void
   }
   const bool tiled_ok = dense_tiled_supports(p);
   // Few output tiles and a long K: split K when the caller's workspace holds the fp32 sums of every slice.
-  if (!unfetchable && !preshuffled && tiled_ok && workspace && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+  if (!unfetchable && tiled_ok && workspace && reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
     const SplitKPlan plan = splitk_plan(M, N, K, device_compute_units());
     if (plan.slices > 1 && workspace_bytes >= (size_t)plan.slices * (size_t)M * (size_t)N * sizeof(float))
       return check_hip(launch_splitk(p, plan, static_cast<float*>(workspace), s), "split-K launch");
@@ -300,6 +300,16 @@ int mslk_amd_f8f8_rowwise_preshuffle(const void* xq, const void* wq_shuffled, co
     return fail("f8f8_rowwise_preshuffle: output dtype code %d is neither bf16 nor fp16", y_dtype);
   return rowwise_impl(y_dtype == MSLK_AMD_DTYPE_F16 ? "f8f8f16_rowwise_preshuffle" : "f8f8bf16_rowwise_preshuffle",
                       y_dtype == MSLK_AMD_DTYPE_F16, 1, xq, wq_shuffled, x_scale, w_scale, bias, bias_dtype, y, M, N, K, nullptr, 0, stream);
+}
+
+int mslk_amd_f8f8_rowwise_preshuffle_workspace(const void* xq, const void* wq_shuffled, const float* x_scale, const float* w_scale,
+                                               const void* bias, int bias_dtype, void* y, int y_dtype, int64_t M, int64_t N,
+                                               int64_t K, void* workspace, size_t workspace_bytes, void* stream) {
+  if (y_dtype != MSLK_AMD_DTYPE_BF16 && y_dtype != MSLK_AMD_DTYPE_F16)
+    return fail("f8f8_rowwise_preshuffle: output dtype code %d is neither bf16 nor fp16", y_dtype);
+  return rowwise_impl(y_dtype == MSLK_AMD_DTYPE_F16 ? "f8f8f16_rowwise_preshuffle" : "f8f8bf16_rowwise_preshuffle",
+                      y_dtype == MSLK_AMD_DTYPE_F16, 1, xq, wq_shuffled, x_scale, w_scale, bias, bias_dtype, y, M, N, K, workspace,
+                      workspace_bytes, stream);
 }
 
 int mslk_amd_preshuffle_b(const void* wq, void* wq_shuffled, int64_t G, int64_t N, int64_t K, void* stream) {

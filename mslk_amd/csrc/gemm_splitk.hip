@@ -15,7 +15,7 @@ constexpr int kGroupM = 4;
 // One workgroup per (tile, slice).  The slices of a tile column sit side by side in the tile list (virtual column
 // s * tiles_n + tn), and the list is dealt to the XCDs in contiguous runs of panels of up to kGroupM row tiles, so the
 // row tiles that read one slice of one weight panel share an L2.
-template <typename TS>
+template <typename TS, bool PS>
 __global__ __launch_bounds__(TS::NTHREADS) void splitk_partial_kernel(GemmProblem p, float* __restrict__ part, int tiles_m,
                                                                       int tiles_n, int slices) {
   constexpr int BM = TS::kBM, BN = TS::kBN;
@@ -34,9 +34,10 @@ __global__ __launch_bounds__(TS::NTHREADS) void splitk_partial_kernel(GemmProble
   const int k0 = step0 * kBK;
   const int klen = (sl == slices - 1 ? p.K : step1 * kBK) - k0;
   const int m0 = tm * BM, n0 = tn * BN;
-  GemmTile<TS, 0> tile;
+  GemmTile<TS, 0, PS> tile;
   tile.out_f16 = 0;
-  tile.run_partial(lds, p.xq + (int64_t)m0 * p.K + k0, p.wq + (int64_t)n0 * p.K + k0,
+  // pre-shuffled weights: a group of 16 rows is contiguous, K step by K step, so byte k0 of its rows lies 16 * k0 bytes in
+  tile.run_partial(lds, p.xq + (int64_t)m0 * p.K + k0, p.wq + (int64_t)n0 * p.K + (PS ? (int64_t)k0 * 16 : (int64_t)k0),
                    part + ((int64_t)sl * p.M + m0) * p.N + n0, p.M - m0, p.N - n0, p.N, klen, (uint32_t)p.K);
 }
 
@@ -88,7 +89,8 @@ template <typename TS>
 hipError_t launch_partial(const GemmProblem& p, float* part, int slices, hipStream_t s) {
   const int tiles_m = (p.M + TS::kBM - 1) / TS::kBM, tiles_n = (p.N + TS::kBN - 1) / TS::kBN;
   const int grid = (tiles_m * tiles_n * slices + kXcds - 1) / kXcds * kXcds;
-  splitk_partial_kernel<TS><<<grid, TS::NTHREADS, 0, s>>>(p, part, tiles_m, tiles_n, slices);
+  if (p.w_preshuffled) splitk_partial_kernel<TS, true><<<grid, TS::NTHREADS, 0, s>>>(p, part, tiles_m, tiles_n, slices);
+  else splitk_partial_kernel<TS, false><<<grid, TS::NTHREADS, 0, s>>>(p, part, tiles_m, tiles_n, slices);
   return hipGetLastError();
 }
 
@@ -125,7 +127,8 @@ SplitKPlan splitk_plan(int64_t M, int64_t N, int64_t K, int cus) {
 }
 
 hipError_t launch_splitk(const GemmProblem& p, const SplitKPlan& plan, float* part, hipStream_t s) {
-  if (dispatch_probe_record("splitk_partial<64,64,waves=4x1,ring=5> slices=%d + splitk_reduce", plan.slices)) return hipSuccess;
+  if (dispatch_probe_record("splitk_partial<64,64,waves=4x1,ring=5>%s slices=%d + splitk_reduce", p.w_preshuffled ? " preshuffled" : "", plan.slices))
+    return hipSuccess;
   const hipError_t e = launch_partial<TileShape<64, 64, 4, 1, 5>>(p, part, plan.slices, s);
   if (e != hipSuccess) return e;
   switch (p.bias_dtype) {

@@ -125,10 +125,15 @@ def _rowwise_impl(XQ, WQ, x_scale, w_scale, bias, use_fast_accum, output=None, o
     bias_ptr, bias_code, _keep = _bias_args(bias, N, XQ.device)
     if preshuffled:
         _check(N % 16 == 0 and K % 64 == 0, f"pre-shuffled weights need N % 16 == 0 and K % 64 == 0, got N={N} K={K}")
+        # few output tiles and a long K: room for the fp32 sums of the K slices, as for row-major weights below
+        wsp_ptr, wsp_bytes = None, _lib.lib().mslk_amd_f8f8bf16_rowwise_workspace_bytes(M, N, K)
+        if wsp_bytes:
+            wsp = torch.empty(wsp_bytes, dtype=torch.uint8, device=XQ.device)
+            wsp_ptr = wsp.data_ptr()
         with _on_device(XQ.device):
-            _lib.check(_lib.lib().mslk_amd_f8f8_rowwise_preshuffle(
+            _lib.check(_lib.lib().mslk_amd_f8f8_rowwise_preshuffle_workspace(
                 XQ.data_ptr(), WQ.data_ptr(), xs.data_ptr(), ws.data_ptr(), bias_ptr, bias_code, Y.data_ptr(),
-                1 if out_dtype == torch.float16 else 0, M, N, K, _stream_ptr(XQ.device)))
+                1 if out_dtype == torch.float16 else 0, M, N, K, wsp_ptr, wsp_bytes, _stream_ptr(XQ.device)))
         return Y
     wsp_ptr, wsp_bytes = None, 0
     if K % 16 or XQ.data_ptr() % 16 or WQ.data_ptr() % 16:

@@ -331,6 +331,31 @@ def test_k_split_exact(M, N, K, bias_dtype, fp16_out):
     _same_bits(y2, want, f"unsplit {M}x{N}x{K}")
 
 
+@pytest.mark.parametrize("fp16_out", [False, True])
+@pytest.mark.parametrize("M,N,K", [(128, 512, 8192), (300, 528, 6208), (96, 2048, 16384)])
+def test_k_split_on_preshuffled_weights_exact(M, N, K, fp16_out):
+    """The K split reads blocked weights as well (a K slice of a 16-row group starts 16 x k0 bytes into the group); the
+    operator passes the workspace, the entry point without one runs the unsplit kernels: the same bits from both."""
+    from mslk_amd import _lib
+    L = _lib.lib()
+    assert L.mslk_amd_debug_dispatch_name(M, N, K, 0, 0, 1, 1).decode().startswith("splitk_partial<64,64,waves=4x1,ring=5> preshuffled")
+    g = torch.Generator().manual_seed(M + N + K)
+    xi, wi, xs, ws = _ints(M, K, g), _ints(N, K, g), _pow2(M, g), _pow2(N, g)
+    bias = torch.randint(-4, 5, (N,), generator=g).float()
+    want = _want(xi, wi, xs, ws, bias, fp16_out)
+    xq, xsd, wsd, bd = xi.to(F8).to(DEV), xs.to(DEV), ws.to(DEV), bias.to(DEV)
+    wshuf = mslk_amd.preshuffle_b_mfma(wi.to(F8).to(DEV))
+    op = torch.ops.mslk.f8f8f16_rowwise_preshuffle if fp16_out else torch.ops.mslk.f8f8bf16_rowwise_preshuffle
+    y = op(xq, wshuf, xsd, wsd, bias=bd)
+    torch.cuda.synchronize()
+    _same_bits(y, want, f"pre-shuffled, split {M}x{N}x{K}")
+    y2 = torch.full((M, N), SENTINEL, dtype=want.dtype, device=DEV)
+    _lib.check(L.mslk_amd_f8f8_rowwise_preshuffle(xq.data_ptr(), wshuf.data_ptr(), xsd.data_ptr(), wsd.data_ptr(), bd.data_ptr(), 1,
+                                                  y2.data_ptr(), 1 if fp16_out else 0, M, N, K, torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    _same_bits(y2, want, f"pre-shuffled, unsplit {M}x{N}x{K}")
+
+
 @pytest.mark.parametrize("M,N,K", [(1, 8192, 5248), (9, 1000, 5376), (16, 4096, 6784), (33, 2560, 5504), (48, 768, 11008), (64, 520, 11264),
                                    (4, 4096, 11008), (20, 1024, 2560)])
 def test_weight_streaming_kernel_exact_on_k_loops_that_do_not_divide_among_its_waves(M, N, K):
